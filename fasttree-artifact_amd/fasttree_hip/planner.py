@@ -1,0 +1,411 @@
+"""Host-side planner of FastTree decode attention: cost model, greedy tree splitter,
+adaptive parallelism loop and the virtual-node ("vnode") metadata builder.
+
+The planner decides, for every radix-tree node, whether its KV is attended together
+with its parent's KV by the node's own requests only (``assignment 1``: the child
+absorbs the ancestor KV, a "Q split") or whether the parent keeps one shared pass
+for all of its requests and the child adds a separate partial (``assignment 0``: a
+"K split" whose price is one more partial to merge).  It then cuts every resulting
+(query set, KV run) pair into vnodes of at most ``Q_TILE`` queries and
+``KV_SPLIT`` tokens and emits the index arrays the two device kernels walk.
+
+Every list this module produces is element-for-element identical to what the
+reference planner produces for the same arguments, including its mutation of the
+``FastTreeParams`` object and the lines it prints.
+
+Reference: kernel_bench/fasttree.py:7-27 (parameters), :30-61 (cost model),
+:64-96 (greedy splitter), :99-296 (adaptive loop and metadata builder).
+"""
+
+from __future__ import annotations
+
+from collections import deque
+from dataclasses import dataclass, field
+from typing import List, Optional, Sequence, Tuple
+
+import numpy as np
+
+#: The reference prints its parallelism estimates, final tile/split sizes and the
+#: per-phase vnode counts on every call.  Set to False to silence the planner.
+VERBOSE = True
+
+#: Number of -1 entries appended to the two entry arrays (kernel_bench/fasttree.py:261-262).
+ENTRY_PADDING = 32
+
+
+class FastTreeParams:
+    """Mutable hyper-parameters of the cost model (kernel_bench/fasttree.py:7-27).
+
+    ``fasttree_preparation`` may replace ``TSQs``/``TSKs`` through the setters while
+    it adapts the tile sizes; callers that reuse one object across trees see that.
+    """
+
+    alpha = 0.66
+    beta = 0.33
+    gamma = 0.1
+    TSQs = [64, 16]
+    TSKs = [32, 128]
+    kv_group_num = 1
+
+    def set_values(self, alpha, beta, gamma):
+        self.alpha, self.beta, self.gamma = alpha, beta, gamma
+
+    def set_kv_group_num(self, kv_group_num):
+        self.kv_group_num = kv_group_num
+
+    def set_q_tile_sizes(self, TSQs):
+        self.TSQs = TSQs
+
+    def set_kv_tile_sizes(self, TSKs):
+        self.TSKs = TSKs
+
+
+# --------------------------------------------------------------------------------------
+# Cost model.  All arithmetic is Python int / IEEE double evaluated left to right,
+# exactly as in the reference, so that near-tie decisions come out the same.
+# --------------------------------------------------------------------------------------
+
+def _CpadQ(TS, N):
+    """Query rows wasted when N queries are tiled by TS (kernel_bench/fasttree.py:30-31).
+    Python's floor modulo makes N == 0 cost nothing: (-1) % TS == TS - 1."""
+    return TS - ((N - 1) % TS + 1)
+
+
+def _CpadK(TS, N):
+    """KV columns wasted when fewer than one tile of keys exists (fasttree.py:34-35)."""
+    return max(0, TS - N)
+
+
+def _Cmm(nQ, nK, params: FastTreeParams):
+    """Padding cost of one (nQ queries x nK keys) contraction (fasttree.py:38-45)."""
+    phase = 0 if nQ > params.TSQs[1] else 1
+    tsq, tsk = params.TSQs[phase], params.TSKs[phase]
+    q_waste = params.alpha * _CpadQ(tsq, nQ) * params.kv_group_num * nK
+    k_waste = params.beta * _CpadK(tsk, nK) * nQ * params.kv_group_num
+    return q_waste + k_waste
+
+
+def _Cred(nQl, params: FastTreeParams, lenl, lenv):
+    """Cost of merging one more partial per query (fasttree.py:48-49)."""
+    return params.gamma * nQl
+
+
+def _SplitQCost(nQcurr, nQl, lenv, lenl, params: FastTreeParams):
+    """Child l leaves with its queries and a private copy of the parent's run
+    (fasttree.py:52-53)."""
+    return _Cmm(nQcurr - nQl, lenv, params) + _Cmm(nQl, lenl + lenv, params)
+
+
+def _SplitKCost(nQcurr, nQl, lenl, lenv, params: FastTreeParams):
+    """Parent run stays shared; child l is a separate partial (fasttree.py:56-61)."""
+    return _Cmm(nQcurr, lenv, params) + _Cmm(nQl, lenl, params) + _Cred(nQl, params, lenl, lenv)
+
+
+def _tree_heuristic(tree_info, params: FastTreeParams) -> List[int]:
+    """Greedy top-down split decision per node (kernel_bench/fasttree.py:64-96).
+
+    Nodes are visited breadth first from node 0, children in ascending id.  While a
+    node's children are scanned, the number of queries still attached to the node
+    shrinks by every child that took the Q split, and a child that took it carries the
+    accumulated run length down to its own children.
+    """
+    count = len(tree_info)
+    children: List[List[int]] = [[] for _ in range(count)]
+    for nid in range(1, count):
+        children[tree_info[nid].parent].append(nid)
+    run_len = [tree_info[nid].seqlen for nid in range(count)]
+
+    assignment = [0] * count
+    pending = deque([0])
+    while pending:
+        v = pending.popleft()
+        attached = len(tree_info[v].requests)
+        lenv = run_len[v]
+        for l in children[v]:
+            nQl = len(tree_info[l].requests)
+            lenl = run_len[l]
+            keep_shared = _SplitKCost(attached, nQl, lenl, lenv, params)
+            go_private = _SplitQCost(attached, nQl, lenv, lenl, params)
+            if keep_shared > go_private:
+                assignment[l] = 1
+                attached -= nQl
+                run_len[l] = lenl + lenv
+            pending.append(l)
+    return assignment
+
+
+# --------------------------------------------------------------------------------------
+# Plan: the pure-host result of the planner (python lists / numpy arrays only).
+# --------------------------------------------------------------------------------------
+
+@dataclass
+class FastTreePlan:
+    """Everything ``fasttree_preparation`` computes before it touches a device."""
+
+    vnode_to_kv_entries: np.ndarray          # int32, padded with ENTRY_PADDING x -1
+    vnode_to_kv_offs: List[int]
+    vnode_to_kv_lens: List[int]
+    vnode_to_q_entries: List[int]
+    vnode_to_q_offs: List[int]
+    vnode_to_q_lens: List[int]
+    req_to_vnode_entries: List[int]          # padded with ENTRY_PADDING x -1
+    req_to_vnode_offs: List[int]
+    req_to_vnode_lens: List[int]
+    phase_node_nums: List[int]
+    phase_node_offsets: List[int]
+    node_assignments: List[int]
+    q_tile_sizes: List[int]                  # final Q_TILE_SIZE_PER_PHASE
+    kv_split_sizes: List[int]                # final KV_SPLIT_SIZE_PER_PHASE
+    parallelisms: List[List[int]] = field(default_factory=list)  # one entry per loop pass
+
+    @property
+    def num_rows(self) -> int:
+        """Rows of the partial-result scratch (``mid_o.shape[0]``)."""
+        return len(self.vnode_to_q_entries)
+
+    @property
+    def num_vnodes(self) -> int:
+        return len(self.vnode_to_q_lens)
+
+
+def _say(*args):
+    if VERBOSE:
+        print(*args)
+
+
+def _requests_per_node(tree_info, assignment) -> List[List[int]]:
+    """Which requests each node's own vnodes serve (fasttree.py:126-141).
+
+    Leaves start with their own request list.  Nodes are then retired in a FIFO order
+    (all leaves in ascending id first, a parent as soon as its last child retires); a
+    retiring node that did not take the Q split hands *all* requests below it to its
+    parent, in retirement order.  The root's parent is -1, which Python resolves to
+    the last list element; the reference does the same and nothing depends on it.
+    """
+    count = len(tree_info)
+    served: List[List[int]] = [[] for _ in range(count)]
+    fifo = deque()
+    for nid in range(count):
+        if tree_info[nid].num_children == 0:
+            fifo.append(nid)
+            served[nid] = list(tree_info[nid].requests)
+    waiting = [tree_info[nid].num_children for nid in range(count)]
+    while fifo:
+        nid = fifo.popleft()
+        up = tree_info[nid].parent
+        if assignment[nid] == 0 and nid != 0:
+            served[up] += tree_info[nid].requests
+        waiting[up] -= 1
+        if waiting[up] == 0:
+            fifo.append(up)
+    return served
+
+
+def _run_chain(tree_info, assignment, nid) -> Tuple[List[int], int]:
+    """Nodes whose KV the vnodes of ``nid`` attend, ancestors first, and the run length
+    (fasttree.py:149-153, :202-210)."""
+    chain = [nid]
+    total = tree_info[nid].seqlen
+    walk = nid
+    while assignment[walk] == 1:
+        walk = tree_info[walk].parent
+        chain.append(walk)
+        total += tree_info[walk].seqlen
+    chain.reverse()
+    return chain, total
+
+
+def _estimate_parallelism(tree_info, assignment, served, q_tiles, kv_splits, num_kv_heads):
+    """Thread-block count per phase the current plan would launch (fasttree.py:143-159)."""
+    blocks = [0, 0]
+    for nid, reqs in enumerate(served):
+        n = len(reqs)
+        if n == 0:
+            continue
+        _, kv_len = _run_chain(tree_info, assignment, nid)
+        phase = 0 if n > q_tiles[1] else 1
+        blocks[phase] += ((kv_len - 1) // kv_splits[phase] + 1) * ((n - 1) // q_tiles[phase] + 1)
+    return [b * num_kv_heads for b in blocks]
+
+
+def fasttree_plan(
+    tree_info,
+    KV_ptrs: Sequence[int],
+    batch_size: int,
+    num_kv_heads: int,
+    KV_SPLIT_SIZES: Sequence[int],
+    para_threshs1: Sequence[int],
+    para_threshs2: Sequence[int],
+    params: FastTreeParams,
+    kv_slot_map: Optional[np.ndarray] = None,
+) -> FastTreePlan:
+    """Run the planner and return host-side lists (kernel_bench/fasttree.py:111-262).
+
+    ``kv_slot_map`` (optional, length ``KV_ptrs[-1]``) maps the logical token position
+    ``KV_ptrs[node] + t`` to the slot of the KV pool that holds it; without it the pool
+    is node-major and the entries are the logical positions themselves, as in the
+    reference's bench.
+    """
+    count = len(tree_info)
+    q_tiles = params.TSQs                       # alias on purpose, as in the reference
+    kv_splits = [KV_SPLIT_SIZES[0], KV_SPLIT_SIZES[0]]
+    history: List[List[int]] = []
+
+    # Up to three passes: (0) shrink KV splits of under-parallel phases, (1) collapse
+    # both phases onto one tile shape if still under-parallel, (2) re-plan with those.
+    for attempt in range(3):
+        assignment = _tree_heuristic(tree_info, params)
+        served = _requests_per_node(tree_info, assignment)
+        para = _estimate_parallelism(tree_info, assignment, served, q_tiles, kv_splits, num_kv_heads)
+        history.append(para)
+        _say("parallelisms:", para)
+        if attempt == 0:
+            starved = [ph for ph in range(2) if 0 < para[ph] < para_threshs1[ph]]
+            for ph in starved:
+                kv_splits[ph] = KV_SPLIT_SIZES[1]
+            if not starved:
+                break
+        elif attempt == 1:
+            if 0 < para[0] < para_threshs2[0]:
+                keep = 1
+            elif 0 < para[1] < para_threshs2[1]:
+                keep = 0
+            else:
+                break
+            q_tiles = [q_tiles[keep], q_tiles[keep]]
+            params.set_q_tile_sizes(q_tiles)
+            params.set_kv_tile_sizes([params.TSKs[keep], params.TSKs[keep]])
+
+    _say(q_tiles)
+    _say(kv_splits)
+
+    ptrs = np.asarray(KV_ptrs, dtype=np.int64)
+    kv_runs: List[np.ndarray] = []
+    kv_total = 0
+    kv_offs: List[int] = []
+    kv_lens: List[int] = []
+    q_entries: List[int] = []
+    q_offs: List[int] = []
+    q_lens: List[int] = []
+
+    q_tile = q_tiles[0]                         # phase-0 tile for every node (fasttree.py:194)
+    for nid in range(count):
+        reqs = served[nid]
+        n = len(reqs)
+        if n == 0:
+            continue
+        kv_split = kv_splits[0 if n > q_tiles[1] else 1]
+        chain, kv_len = _run_chain(tree_info, assignment, nid)
+        run_base = kv_total
+        for member in chain:
+            kv_runs.append(np.arange(ptrs[member], ptrs[member + 1], dtype=np.int64))
+        kv_total += kv_len
+
+        for kv_lo in range(0, kv_len, kv_split):
+            row_base = len(q_entries)
+            q_entries.extend(reqs)              # one scratch row per (request, kv split)
+            span = min(kv_lo + kv_split, kv_len) - kv_lo
+            for q_lo in range(0, n, q_tile):
+                kv_offs.append(run_base + kv_lo)
+                kv_lens.append(span)
+                q_offs.append(row_base + q_lo)
+                q_lens.append(min(q_lo + q_tile, n) - q_lo)
+
+    rows_of_req: List[List[int]] = [[] for _ in range(batch_size)]
+    for row, req in enumerate(q_entries):
+        rows_of_req[req].append(row)
+    req_offs: List[int] = []
+    req_lens: List[int] = []
+    req_entries: List[int] = []
+    for rows in rows_of_req:
+        req_offs.append(len(req_entries))
+        req_lens.append(len(rows))
+        req_entries.extend(rows)
+
+    # Stable partition: vnodes wider than the small tile run first (phase 0).
+    small = q_tiles[1]
+    wide = [v for v, n in enumerate(q_lens) if n > small]
+    narrow = [v for v, n in enumerate(q_lens) if n <= small]
+    _say("Above threshold: ", len(wide))
+    _say("Below threshold: ", len(narrow))
+    order = wide + narrow
+
+    logical = np.concatenate(kv_runs) if kv_runs else np.zeros(0, dtype=np.int64)
+    if kv_slot_map is not None:
+        logical = np.asarray(kv_slot_map)[logical]
+    padded = np.concatenate([logical, np.full(ENTRY_PADDING, -1, dtype=np.int64)]).astype(np.int32)
+
+    return FastTreePlan(
+        vnode_to_kv_entries=padded,
+        vnode_to_kv_offs=[kv_offs[v] for v in order],
+        vnode_to_kv_lens=[kv_lens[v] for v in order],
+        vnode_to_q_entries=q_entries,
+        vnode_to_q_offs=[q_offs[v] for v in order],
+        vnode_to_q_lens=[q_lens[v] for v in order],
+        req_to_vnode_entries=req_entries + [-1] * ENTRY_PADDING,
+        req_to_vnode_offs=req_offs,
+        req_to_vnode_lens=req_lens,
+        phase_node_nums=[len(wide), len(narrow)],
+        phase_node_offsets=[0, len(wide)],
+        node_assignments=assignment,
+        q_tile_sizes=list(q_tiles),
+        kv_split_sizes=kv_splits,
+        parallelisms=history,
+    )
+
+
+def fasttree_preparation(
+    tree_info,
+    KV_ptrs,
+    batch_size,
+    num_qo_heads,
+    num_kv_heads,
+    head_dim,
+    KV_SPLIT_SIZES,
+    para_threshs1,
+    para_threshs2,
+    params: FastTreeParams,
+    *,
+    device="cuda",
+    kv_slot_map=None,
+):
+    """Drop-in for kernel_bench/fasttree.py:99-296: plan on the host, then place the nine
+    int32 index arrays and the two fp32 partial-result buffers on ``device``.
+
+    Returns ``((vnode_to_kv_entries, vnode_to_kv_offs, vnode_to_kv_lens,
+    vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, req_to_vnode_entries,
+    req_to_vnode_offs, req_to_vnode_lens, mid_o, mid_lse, phase_node_nums,
+    phase_node_offsets), node_assignments)``.  The keyword-only arguments do not exist
+    in the reference: ``device`` defaults to the reference's hard-wired "cuda";
+    ``kv_slot_map`` is described in :func:`fasttree_plan`.
+    """
+    import torch
+
+    plan = fasttree_plan(
+        tree_info, KV_ptrs, batch_size, num_kv_heads,
+        KV_SPLIT_SIZES, para_threshs1, para_threshs2, params, kv_slot_map=kv_slot_map,
+    )
+
+    def put(values):
+        host = torch.from_numpy(np.ascontiguousarray(np.asarray(values, dtype=np.int32)))
+        return host.to(device)
+
+    rows = plan.num_rows
+    mid_o = torch.empty((rows, num_qo_heads, head_dim), dtype=torch.float32, device=device)
+    mid_lse = torch.empty((rows, num_qo_heads), dtype=torch.float32, device=device)
+    aux = (
+        put(plan.vnode_to_kv_entries),
+        put(plan.vnode_to_kv_offs),
+        put(plan.vnode_to_kv_lens),
+        put(plan.vnode_to_q_entries),
+        put(plan.vnode_to_q_offs),
+        put(plan.vnode_to_q_lens),
+        put(plan.req_to_vnode_entries),
+        put(plan.req_to_vnode_offs),
+        put(plan.req_to_vnode_lens),
+        mid_o,
+        mid_lse,
+        plan.phase_node_nums,
+        plan.phase_node_offsets,
+    )
+    return aux, plan.node_assignments

@@ -1,0 +1,119 @@
+/*
+ * C ABI of libfasttree_hip.so: FastTree tree-structured decode attention for AMD
+ * Instinct MI355X (gfx950).
+ *
+ * The functions below are what a foreign-function binding of the reference's decode
+ * path would bind.  They take plain device pointers, element strides and sizes; they
+ * allocate nothing, keep no pointer after returning, never synchronise the device and
+ * enqueue all work on the HIP stream that is passed in.  Every function returns
+ * FT_OK (0) or a negative FT_ERR_* code; ft_error_string() names a code.
+ *
+ * Conventions shared by all entry points
+ *   - dtype: FT_DTYPE_F16 or FT_DTYPE_BF16, the element type of q, k, v and o.
+ *   - q, o:  [batch, Hq, D]; k, v: [slots, Hkv, D]; the last dimension is contiguous,
+ *     the two outer strides are given in elements and must be multiples of 8, and the
+ *     base pointers must be 16-byte aligned.  K and V are separate allocations.
+ *   - mid_o [rows, Hq, D] and mid_lse [rows, Hq] are caller-owned fp32 scratch; stage 1
+ *     overwrites them with the per-vnode partial result normalised by its own soft-max
+ *     sum and with log-sum-exp of the scaled scores (natural log).  mid_o strides must
+ *     be multiples of 4, the head stride of mid_lse is 1.
+ *   - index arrays are contiguous int32 in device memory.  No element past the ranges
+ *     named by the offset/length arrays is ever read.
+ *   - D in {32, 64, 128, 256}; Hq = Hkv * g with 1 <= g <= 64; sm_scale > 0.
+ */
+#ifndef FASTTREE_HIP_H_
+#define FASTTREE_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ihipStream_t* ft_stream_t; /* a hipStream_t; NULL = the null stream */
+
+enum { FT_DTYPE_F16 = 0, FT_DTYPE_BF16 = 1 };
+
+enum {
+  FT_OK = 0,
+  FT_ERR_NULL_POINTER = -1,
+  FT_ERR_DTYPE = -2,
+  FT_ERR_HEAD_DIM = -3,      /* reference: assert Lk in {16,32,64,128,256}, kernel_bench/fasttree.py:439 */
+  FT_ERR_GROUP = -4,
+  FT_ERR_ALIGNMENT = -5,
+  FT_ERR_ARGUMENT = -6,
+  FT_ERR_LAUNCH = -7
+};
+
+/* Library version string, e.g. "fasttree_hip 0.1 (gfx950)". */
+const char* ft_version(void);
+
+/* Human-readable name of a return code. */
+const char* ft_error_string(int code);
+
+/*
+ * Stage 1 for one phase: the partial attention of every vnode in
+ * [vnode_begin, vnode_begin + vnode_count) against its KV slice, for all KV heads.
+ * Replaces one launch of _fwd_fasttree_decode_stage1 by _fasttree_decode_stage1
+ * (kernel_bench/fasttree.py:299-413, :443-479).  q_tile is the phase's query tile
+ * (requests per vnode the planner used); vnodes with more requests are still computed
+ * in full.  kv_tile is accepted for signature parity and does not change the result.
+ */
+int ft_stage1(const void* q, const void* k, const void* v,
+              int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+              const int32_t* vnode_to_kv_entries, const int32_t* vnode_to_kv_offs,
+              const int32_t* vnode_to_kv_lens, const int32_t* vnode_to_q_entries,
+              const int32_t* vnode_to_q_offs, const int32_t* vnode_to_q_lens,
+              int vnode_begin, int vnode_count, int num_kv_heads, int kv_group_num, int head_dim,
+              int q_tile, int kv_tile, float sm_scale,
+              float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
+              int dtype, ft_stream_t stream);
+
+/*
+ * Stage 2: per (request, query head) log-sum-exp weighted merge of the request's
+ * partial rows into o.  Replaces _fwd_fasttree_decoding_stage2 / _fasttree_decode_stage2
+ * (kernel_bench/fasttree.py:482-579).
+ */
+int ft_stage2(const int32_t* req_to_vnode_entries, const int32_t* req_to_vnode_offs,
+              const int32_t* req_to_vnode_lens,
+              const float* mid_o, int64_t so0, int64_t so1, const float* mid_lse, int64_t sl0,
+              void* o, int64_t oo0, int64_t oo1,
+              int batch_size, int num_qo_heads, int head_dim, int dtype, ft_stream_t stream);
+
+/*
+ * The whole decode call: stage 1 for both phases, then stage 2.  Replaces
+ * fasttree_decode (kernel_bench/fasttree.py:582-642); phase_* are its four 2-element
+ * python lists.
+ */
+int ft_decode(const void* q, const void* k, const void* v, void* o,
+              int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+              int64_t oo0, int64_t oo1,
+              const int32_t* vnode_to_kv_entries, const int32_t* vnode_to_kv_offs,
+              const int32_t* vnode_to_kv_lens, const int32_t* vnode_to_q_entries,
+              const int32_t* vnode_to_q_offs, const int32_t* vnode_to_q_lens,
+              const int32_t* req_to_vnode_entries, const int32_t* req_to_vnode_offs,
+              const int32_t* req_to_vnode_lens,
+              float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
+              const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
+              const int32_t phase_q_tile_sizes[2], const int32_t phase_kv_tile_sizes[2],
+              int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
+              float sm_scale, int dtype, ft_stream_t stream);
+
+/*
+ * Decode attention without prefix sharing over a per-request gathered, padded cache
+ * k_cache, v_cache [batch, max_seqlen, Hkv, D] (contiguous) with cache_seqlens [batch]:
+ * the layout the reference's comparison engines read (kernel_bench/flash_attn_wrap.py:36-70,
+ * flashinfer_wrap.py:13-16).  Each request's sequence is cut into ceil(max_seqlen /
+ * kv_split) pieces; mid_o / mid_lse need batch * ceil(max_seqlen / kv_split) rows.
+ */
+int ft_gathered_decode(const void* q, const void* k_cache, const void* v_cache,
+                       const int32_t* cache_seqlens, void* o,
+                       int64_t sq0, int64_t sq1, int64_t oo0, int64_t oo1,
+                       int batch_size, int max_seqlen, int num_qo_heads, int num_kv_heads,
+                       int head_dim, int kv_split, float sm_scale,
+                       float* mid_o, float* mid_lse, int dtype, ft_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FASTTREE_HIP_H_ */
