@@ -1,0 +1,695 @@
+// FastTree tree-structured decode attention for gfx950 (MI355X): the two device kernels
+// and the C ABI declared in include/fasttree_hip.h.
+//
+// Stage 1 computes, for every virtual node (a set of <= Q_TILE requests that share one run
+// of KV tokens) and every KV head, the soft-max partial of those requests' query heads
+// over that run.  All query rows of a vnode (requests x GQA group) form the N side of
+// 16x16x32 MFMA tiles; the gathered K rows are the M side of S^T = K Q^T and the gathered
+// V rows are read back from LDS transposed (ds_read_b64_tr_b16) as the M side of
+// O^T = V^T P^T, so the probabilities go from the first contraction's accumulators
+// straight into the second contraction's B operand without leaving registers.
+//
+// Stage 2 merges each request's partials with their log-sum-exp weights using shuffles
+// inside a group of D/4 lanes.
+//
+// Reference for the arithmetic: kernel_bench/fasttree.py:299-413 (stage 1), :482-546
+// (stage 2), :582-642 (the call that chains them).
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/fasttree_hip.h"
+
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+constexpr int kWavesPerBlock = 4;
+constexpr int kBlock = kWave * kWavesPerBlock;
+constexpr int kTileTokens = 32;          // KV tokens per inner step (two 16-token MFMA row blocks)
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// ---------------------------------------------------------------------------------------
+// Element-type traits: the 16-bit storage type only matters at the MFMA call and where
+// fp32 probabilities / outputs are rounded to it.
+// ---------------------------------------------------------------------------------------
+struct F16 {
+  static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ unsigned pack2(float lo, float hi) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    h2 v = {(_Float16)lo, (_Float16)hi};
+    return __builtin_bit_cast(unsigned, v);
+  }
+};
+struct BF16 {
+  static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ unsigned pack2(float lo, float hi) {
+    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+    b2 v = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(unsigned, v);
+  }
+};
+
+// Wave-wide exchange helpers.  v_permlane{16,32}_swap with both operands equal to x
+// return (x of the lower half, x of the upper half) of each 32-lane / 64-lane group.
+__device__ __forceinline__ float xor16_max(float x) {
+  auto r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, x), false, false);
+  return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+}
+__device__ __forceinline__ float xor32_max(float x) {
+  auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, x), false, false);
+  return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+}
+__device__ __forceinline__ float xor16_sum(float x) {
+  auto r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, x), false, false);
+  return __builtin_bit_cast(float, r[0]) + __builtin_bit_cast(float, r[1]);
+}
+__device__ __forceinline__ float xor32_sum(float x) {
+  auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, x), false, false);
+  return __builtin_bit_cast(float, r[0]) + __builtin_bit_cast(float, r[1]);
+}
+// Orders this wave's LDS traffic around a point where lanes read what other lanes of the
+// same wave wrote.  LDS executes one wave's instructions in order, so no wait is needed;
+// the fences only stop the compiler from moving accesses across.
+__device__ __forceinline__ void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+__device__ __forceinline__ float scale_from(float m_part, float m_all) {
+  return (m_part == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_part - m_all);
+}
+
+struct Stage1Args {
+  const char* q;
+  const char* k;
+  const char* v;
+  int64_t sq0, sq1, sk0, sk1, sv0, sv1;  // element strides
+  const int32_t* kv_entries;
+  const int32_t* kv_offs;
+  const int32_t* kv_lens;
+  const int32_t* q_entries;
+  const int32_t* q_offs;
+  const int32_t* q_lens;
+  int vnode_begin, vnode_count;
+  int g;
+  float scale_log2;  // sm_scale * log2(e)
+  float* mid_o;
+  int64_t so0, so1;
+  float* mid_lse;
+  int64_t sl0;
+  // gathered (no-sharing) mode: vnode = (request, split) over a padded per-request cache
+  const int32_t* cache_seqlens;
+  int max_seqlen, kv_split, nsplit;
+};
+
+// How a kernel instance finds its vnode's slices.
+struct VnodeView {
+  int q_off;       // first scratch row
+  int q_len;       // requests in this vnode
+  int kv_len;      // tokens in the run
+  int64_t kv_base; // tree mode: index into kv_entries; gathered mode: first cache row
+};
+
+template <bool GATHERED>
+__device__ __forceinline__ VnodeView load_vnode(const Stage1Args& a, int vnode) {
+  VnodeView w;
+  if constexpr (GATHERED) {
+    int req = vnode / a.nsplit, split = vnode - req * a.nsplit;
+    int len = a.cache_seqlens[req] - split * a.kv_split;
+    w.kv_len = len < 0 ? 0 : (len > a.kv_split ? a.kv_split : len);
+    w.kv_base = (int64_t)req * a.max_seqlen + (int64_t)split * a.kv_split;
+    w.q_off = vnode;
+    w.q_len = 1;
+  } else {
+    w.q_off = a.q_offs[vnode];
+    w.q_len = a.q_lens[vnode];
+    w.kv_len = a.kv_lens[vnode];
+    w.kv_base = a.kv_offs[vnode];
+  }
+  return w;
+}
+
+// Per-wave LDS staging of one 32-token tile.  Row pitches are chosen for the two read
+// patterns: K rows are read 16 B per lane by 16 different rows at a time (pitch = 4 dwords
+// mod 64 banks), V rows are read by ds_read_b64_tr_b16, where 16 lanes cover 4 rows x 32 B
+// (pitch = 8 dwords mod 32 banks).
+template <int D> struct TileGeom {
+  static constexpr int kRowBytes = D * 2;
+  static constexpr int kPitchK = kRowBytes + 16;
+  static constexpr int kPitchV = kRowBytes + 32;
+  static constexpr int kBytesK = kTileTokens * kPitchK;
+  static constexpr int kBytesV = kTileTokens * kPitchV;
+  static constexpr int kBytes = kBytesK + kBytesV;     // per wave
+  static constexpr int kLanesPerRow = D / 8;           // 16-byte chunks in a row
+  static constexpr int kRowsPerLoad = kWave / kLanesPerRow;
+  static constexpr int kLoads = kTileTokens / kRowsPerLoad;
+};
+
+// Running soft-max state of one wave for NQB blocks of 16 query rows.  Accumulators are
+// O^T tiles: lane l holds o[qb][db][j] = O[row 16*qb + l%16][dim 16*db + 4*(l/16) + j].
+template <int D, int NQB> struct WaveState {
+  f32x4 o[NQB][D / 16];
+  float m[NQB];  // running max of scaled scores, log2 domain, identical in the 4 lanes of a row
+  float l[NQB];  // running sum of this lane's own probabilities (reduced over lanes at the end)
+};
+
+// One wave attends NQB*16 query rows to tokens [tile0*32, ...) in steps of tile_step tiles.
+template <typename E, int D, int NQB, bool GATHERED>
+__device__ __forceinline__ void wave_attend(const Stage1Args& a, const VnodeView& vn, int kvh, int row0,
+                                            int tile0, int tile_step, char* lds, WaveState<D, NQB>& st) {
+  using G = TileGeom<D>;
+  constexpr int KS = D / 32, DB = D / 16;
+  const int lane = threadIdx.x & 63;
+  const int p = lane & 15, c = lane >> 4;
+  char* ldsK = lds;
+  char* ldsV = lds + G::kBytesK;
+
+  // ---- query fragments (B operand of S^T = K Q^T): row 16*qb + p, dims 32*ks + 8*c .. +7
+  u32x4 qf[NQB][KS];
+  const int rows_total = vn.q_len * a.g;
+#pragma unroll
+  for (int qb = 0; qb < NQB; ++qb) {
+    const int r = row0 + 16 * qb + p;
+    const bool ok = r < rows_total;
+    const int ri = ok ? r / a.g : 0;
+    const int rj = ok ? r - ri * a.g : 0;
+    const int64_t entry = ok ? (GATHERED ? (int64_t)(vn.q_off / a.nsplit) : (int64_t)a.q_entries[vn.q_off + ri]) : 0;
+    const char* src = a.q + 2 * (entry * a.sq0 + (int64_t)(kvh * a.g + rj) * a.sq1 + 8 * c);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      u32x4 z = {0u, 0u, 0u, 0u};
+      qf[qb][ks] = ok ? *reinterpret_cast<const u32x4*>(src + 64 * ks) : z;
+    }
+  }
+
+#pragma unroll
+  for (int qb = 0; qb < NQB; ++qb) {
+    st.m[qb] = -INFINITY;
+    st.l[qb] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) st.o[qb][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  const int ntiles = (vn.kv_len + kTileTokens - 1) / kTileTokens;
+  if (tile0 >= ntiles) return;
+
+  // ---- global -> register prefetch of one tile (rows by 16-byte chunks, coalesced per row)
+  const int ld_row = lane / G::kLanesPerRow, ld_chunk = lane % G::kLanesPerRow;
+  u32x4 kreg[G::kLoads], vreg[G::kLoads];
+  auto fetch = [&](int tile) {
+#pragma unroll
+    for (int i = 0; i < G::kLoads; ++i) {
+      const int t = tile * kTileTokens + i * G::kRowsPerLoad + ld_row;
+      u32x4 z = {0u, 0u, 0u, 0u};
+      kreg[i] = z;
+      vreg[i] = z;
+      if (t < vn.kv_len) {
+        const int64_t slot = GATHERED ? (vn.kv_base + t) : (int64_t)a.kv_entries[vn.kv_base + t];
+        kreg[i] = *reinterpret_cast<const u32x4*>(a.k + 2 * (slot * a.sk0 + (int64_t)kvh * a.sk1) + 16 * ld_chunk);
+        vreg[i] = *reinterpret_cast<const u32x4*>(a.v + 2 * (slot * a.sv0 + (int64_t)kvh * a.sv1) + 16 * ld_chunk);
+      }
+    }
+  };
+  fetch(tile0);
+
+  for (int tile = tile0; tile < ntiles; tile += tile_step) {
+    // registers -> this wave's LDS tile
+#pragma unroll
+    for (int i = 0; i < G::kLoads; ++i) {
+      const int row = i * G::kRowsPerLoad + ld_row;
+      *reinterpret_cast<u32x4*>(ldsK + row * G::kPitchK + 16 * ld_chunk) = kreg[i];
+      *reinterpret_cast<u32x4*>(ldsV + row * G::kPitchV + 16 * ld_chunk) = vreg[i];
+    }
+    wave_lds_fence();
+    if (tile + tile_step < ntiles) fetch(tile + tile_step);
+
+    // ---- S^T = K Q^T : s[tb][qb][j] = score(token 16*tb + 4*c + j, row 16*qb + p)
+    f32x4 s[2][NQB];
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb) {
+#pragma unroll
+      for (int qb = 0; qb < NQB; ++qb) s[tb][qb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const u32x4 kf = *reinterpret_cast<const u32x4*>(ldsK + (16 * tb + p) * G::kPitchK + 64 * ks + 16 * c);
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb) s[tb][qb] = E::mfma(kf, qf[qb][ks], s[tb][qb]);
+      }
+    }
+
+    const int valid = vn.kv_len - tile * kTileTokens;  // tokens of this tile that exist
+    const float sc = a.scale_log2;
+    u32x4 pf[NQB];
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) {
+      float x[8];
+#pragma unroll
+      for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          float val = s[tb][qb][j] * sc;
+          if (valid < kTileTokens && 16 * tb + 4 * c + j >= valid) val = -INFINITY;
+          x[4 * tb + j] = val;
+        }
+      float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+      mx = xor32_max(xor16_max(mx));
+      const float m_old = st.m[qb];
+      const float m_new = fmaxf(m_old, mx);  // finite: every tile holds at least one token
+      float sum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        x[i] = __builtin_amdgcn_exp2f(x[i] - m_new);
+        sum += x[i];
+      }
+      if (__builtin_amdgcn_ballot_w64(m_new > m_old)) {  // wave-uniform: rescale only when a max moved
+        const float alpha = __builtin_amdgcn_exp2f(m_old - m_new);
+        st.l[qb] *= alpha;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) st.o[qb][db] *= alpha;
+      }
+      st.l[qb] += sum;
+      st.m[qb] = m_new;
+      pf[qb] = u32x4{E::pack2(x[0], x[1]), E::pack2(x[2], x[3]), E::pack2(x[4], x[5]), E::pack2(x[6], x[7])};
+    }
+
+    // ---- O^T += V^T P^T : A operand rows = dims 16*db + p, k slots = the 8 tokens this lane's P holds
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const char* va = ldsV + (4 * c + (p >> 2)) * G::kPitchV + 2 * (16 * db + 4 * (p & 3));
+      const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) i16x4*)(va));
+      const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) i16x4*)(va + 16 * G::kPitchV));
+      const u32x2 lo2 = __builtin_bit_cast(u32x2, lo), hi2 = __builtin_bit_cast(u32x2, hi);
+      const u32x4 vf = {lo2[0], lo2[1], hi2[0], hi2[1]};
+#pragma unroll
+      for (int qb = 0; qb < NQB; ++qb) st.o[qb][db] = E::mfma(vf, pf[qb], st.o[qb][db]);
+    }
+    wave_lds_fence();
+  }
+
+  // every lane of a row now gets the row's full probability sum
+#pragma unroll
+  for (int qb = 0; qb < NQB; ++qb) st.l[qb] = xor32_sum(xor16_sum(st.l[qb]));
+}
+
+template <int D, int NQB>
+__device__ __forceinline__ void write_partials(const Stage1Args& a, const VnodeView& vn, int kvh, int row0,
+                                               const WaveState<D, NQB>& st) {
+  constexpr int DB = D / 16;
+  const int lane = threadIdx.x & 63;
+  const int p = lane & 15, c = lane >> 4;
+  const int rows_total = vn.q_len * a.g;
+#pragma unroll
+  for (int qb = 0; qb < NQB; ++qb) {
+    const int r = row0 + 16 * qb + p;
+    if (r >= rows_total) continue;
+    const int ri = r / a.g, rj = r - ri * a.g;
+    const int64_t row = vn.q_off + ri;
+    const int head = kvh * a.g + rj;
+    const float l = st.l[qb];
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    float* dst = a.mid_o + row * a.so0 + (int64_t)head * a.so1 + 4 * c;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) *reinterpret_cast<f32x4*>(dst + 16 * db) = st.o[qb][db] * inv;
+    if (c == 0) a.mid_lse[row * a.sl0 + head] = l > 0.f ? (__builtin_amdgcn_logf(l) + st.m[qb]) * kLn2 : -INFINITY;
+  }
+}
+
+// SPLIT_WAVES = true : one block per (vnode, kv head); its 4 waves take every 4th KV tile and
+//                      their states are merged through LDS (wide vnodes, long runs).
+// SPLIT_WAVES = false: one wave per (vnode, kv head), 4 vnodes per block (narrow vnodes).
+template <typename E, int D, int NQB, bool SPLIT_WAVES, bool GATHERED>
+__global__ void __launch_bounds__(kBlock) stage1_kernel(Stage1Args a) {
+  using G = TileGeom<D>;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int kvh = blockIdx.y;
+  char* my_lds = smem + wave * G::kBytes;
+
+  if constexpr (!SPLIT_WAVES) {
+    const int local = blockIdx.x * kWavesPerBlock + wave;
+    if (local >= a.vnode_count) return;
+    const VnodeView vn = load_vnode<GATHERED>(a, a.vnode_begin + local);
+    const int rows_total = vn.q_len * a.g;
+    for (int row0 = 0; row0 < rows_total; row0 += 16 * NQB) {
+      WaveState<D, NQB> st;
+      wave_attend<E, D, NQB, GATHERED>(a, vn, kvh, row0, 0, 1, my_lds, st);
+      write_partials<D, NQB>(a, vn, kvh, row0, st);
+    }
+  } else {
+    const VnodeView vn = load_vnode<GATHERED>(a, a.vnode_begin + blockIdx.x);
+    const int rows_total = vn.q_len * a.g;
+    constexpr int NV = NQB * (D / 16) * 4 + 2 * NQB;  // floats of state per lane
+    float* xchg = reinterpret_cast<float*>(smem);
+    for (int row0 = 0; row0 < rows_total; row0 += 16 * NQB) {
+      WaveState<D, NQB> st;
+      wave_attend<E, D, NQB, GATHERED>(a, vn, kvh, row0, wave, kWavesPerBlock, my_lds, st);
+      // pairwise merge: waves {2,3} -> {0,1}, then wave 1 -> wave 0, through the staging LDS
+#pragma unroll
+      for (int half = 2; half >= 1; half >>= 1) {
+        __syncthreads();
+        if (wave >= half && wave < 2 * half) {
+          float* dst = xchg + (size_t)(wave - half) * NV * kWave + lane;
+          int n = 0;
+#pragma unroll
+          for (int qb = 0; qb < NQB; ++qb) {
+            dst[(n++) * kWave] = st.m[qb];
+            dst[(n++) * kWave] = st.l[qb];
+#pragma unroll
+            for (int db = 0; db < D / 16; ++db)
+#pragma unroll
+              for (int j = 0; j < 4; ++j) dst[(n++) * kWave] = st.o[qb][db][j];
+          }
+        }
+        __syncthreads();
+        if (wave < half) {
+          const float* src = xchg + (size_t)wave * NV * kWave + lane;
+          int n = 0;
+#pragma unroll
+          for (int qb = 0; qb < NQB; ++qb) {
+            const float m2 = src[(n++) * kWave];
+            const float l2 = src[(n++) * kWave];
+            const float m = fmaxf(st.m[qb], m2);
+            const float a1 = scale_from(st.m[qb], m), a2 = scale_from(m2, m);
+            st.l[qb] = st.l[qb] * a1 + l2 * a2;
+            st.m[qb] = m;
+#pragma unroll
+            for (int db = 0; db < D / 16; ++db)
+#pragma unroll
+              for (int j = 0; j < 4; ++j) st.o[qb][db][j] = st.o[qb][db][j] * a1 + src[(n++) * kWave] * a2;
+          }
+        }
+      }
+      if (wave == 0) write_partials<D, NQB>(a, vn, kvh, row0, st);
+      __syncthreads();  // staging LDS is reused by the next row chunk
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Stage 2
+// ---------------------------------------------------------------------------------------
+struct Stage2Args {
+  const int32_t* req_entries;
+  const int32_t* req_offs;
+  const int32_t* req_lens;
+  const float* mid_o;
+  int64_t so0, so1;
+  const float* mid_lse;
+  int64_t sl0;
+  char* o;
+  int64_t oo0, oo1;
+  int batch, hq;
+  int nsplit;  // > 0: gathered mode, request r owns rows [r*nsplit, (r+1)*nsplit)
+};
+
+template <int WIDTH> __device__ __forceinline__ float group_max(float x) {
+#pragma unroll
+  for (int d = WIDTH / 2; d >= 1; d >>= 1) x = fmaxf(x, __shfl_xor(x, d, WIDTH));
+  return x;
+}
+template <int WIDTH> __device__ __forceinline__ float group_sum(float x) {
+#pragma unroll
+  for (int d = WIDTH / 2; d >= 1; d >>= 1) x += __shfl_xor(x, d, WIDTH);
+  return x;
+}
+
+// A group of D/4 lanes owns one (request, head): lane i fetches the row index and the
+// log-sum-exp of partial i, the group reduces max and weight sum with shuffles, then every
+// lane accumulates its own 4 output dims over the partials, taking weight and row index of
+// partial i from lane i.
+template <typename E, int D>
+__global__ void __launch_bounds__(kBlock) stage2_kernel(Stage2Args a) {
+  constexpr int LPH = D / 4;
+  constexpr int HPB = kBlock / LPH;
+  const int grp = threadIdx.x / LPH, gl = threadIdx.x % LPH;
+  const int req = blockIdx.x;
+  const int head = blockIdx.y * HPB + grp;
+  if (head >= a.hq) return;
+  const int off = a.nsplit > 0 ? req * a.nsplit : a.req_offs[req];
+  const int n = a.nsplit > 0 ? a.nsplit : a.req_lens[req];
+
+  float m_run = -INFINITY, l_run = 0.f;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int base = 0; base < n; base += LPH) {
+    const int cnt = min(LPH, n - base);
+    int my_row = -1;
+    float my_lse = -INFINITY;
+    if (gl < cnt) {
+      my_row = a.nsplit > 0 ? off + base + gl : a.req_entries[off + base + gl];
+      my_lse = a.mid_lse[(int64_t)my_row * a.sl0 + head];
+    }
+    const float m_new = fmaxf(m_run, group_max<LPH>(my_lse));
+    const float w = (my_lse == -INFINITY) ? 0.f : __expf(my_lse - m_new);
+    const float keep = (m_run == -INFINITY) ? 0.f : __expf(m_run - m_new);
+    l_run = l_run * keep + group_sum<LPH>(w);
+    acc *= keep;
+    m_run = m_new;
+#pragma unroll 4
+    for (int i = 0; i < cnt; ++i) {
+      const float wi = __shfl(w, i, LPH);
+      const int ri = __shfl(my_row, i, LPH);
+      if (wi != 0.f) {
+        const f32x4 part = *reinterpret_cast<const f32x4*>(a.mid_o + (int64_t)ri * a.so0 + (int64_t)head * a.so1 + 4 * gl);
+        acc += part * wi;
+      }
+    }
+  }
+  const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+  acc *= inv;
+  u32x2 out = {E::pack2(acc[0], acc[1]), E::pack2(acc[2], acc[3])};
+  *reinterpret_cast<u32x2*>(a.o + 2 * ((int64_t)req * a.oo0 + (int64_t)head * a.oo1 + 4 * gl)) = out;
+}
+
+// ---------------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------------
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <typename E, int D, int NQB, bool SPLIT, bool GATHERED>
+int launch_stage1_inst(const Stage1Args& a, int hkv, hipStream_t stream) {
+  const size_t lds = (size_t)kWavesPerBlock * TileGeom<D>::kBytes;
+  auto kern = stage1_kernel<E, D, NQB, SPLIT, GATHERED>;
+  static bool configured = false;  // raising the dynamic LDS limit is idempotent
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+      (void)hipGetLastError();
+      return FT_ERR_LAUNCH;
+    }
+    configured = true;
+  }
+  const unsigned gx = SPLIT ? (unsigned)a.vnode_count : (unsigned)((a.vnode_count + kWavesPerBlock - 1) / kWavesPerBlock);
+  hipLaunchKernelGGL(kern, dim3(gx, (unsigned)hkv, 1), dim3(kBlock, 1, 1), lds, stream, a);
+  return hipGetLastError() == hipSuccess ? FT_OK : FT_ERR_LAUNCH;
+}
+
+template <typename E, int D, bool GATHERED>
+int launch_stage1_d(const Stage1Args& a, int hkv, int rows_per_vnode, hipStream_t stream) {
+  // Row blocks per wave: enough for the phase's tile, at most 64 rows (wider vnodes loop).
+  constexpr int kMaxNqb = D > 128 ? 2 : 4;
+  if (rows_per_vnode <= 16) return launch_stage1_inst<E, D, 1, false, GATHERED>(a, hkv, stream);
+  if (rows_per_vnode <= 32 || kMaxNqb == 2) return launch_stage1_inst<E, D, 2, true, GATHERED>(a, hkv, stream);
+  return launch_stage1_inst<E, D, kMaxNqb, true, GATHERED>(a, hkv, stream);
+}
+
+template <bool GATHERED>
+int launch_stage1(const Stage1Args& a, int hkv, int d, int rows_per_vnode, int dtype, hipStream_t stream) {
+#define FT_DISPATCH_D(E)                                                                  \
+  switch (d) {                                                                            \
+    case 32: return launch_stage1_d<E, 32, GATHERED>(a, hkv, rows_per_vnode, stream);     \
+    case 64: return launch_stage1_d<E, 64, GATHERED>(a, hkv, rows_per_vnode, stream);     \
+    case 128: return launch_stage1_d<E, 128, GATHERED>(a, hkv, rows_per_vnode, stream);   \
+    case 256: return launch_stage1_d<E, 256, GATHERED>(a, hkv, rows_per_vnode, stream);   \
+    default: return FT_ERR_HEAD_DIM;                                                      \
+  }
+  if (dtype == FT_DTYPE_F16) { FT_DISPATCH_D(F16) }
+  if (dtype == FT_DTYPE_BF16) { FT_DISPATCH_D(BF16) }
+#undef FT_DISPATCH_D
+  return FT_ERR_DTYPE;
+}
+
+template <typename E, int D>
+int launch_stage2_inst(const Stage2Args& a, hipStream_t stream) {
+  constexpr int HPB = kBlock / (D / 4);
+  hipLaunchKernelGGL((stage2_kernel<E, D>), dim3((unsigned)a.batch, (unsigned)((a.hq + HPB - 1) / HPB), 1),
+                     dim3(kBlock, 1, 1), 0, stream, a);
+  return hipGetLastError() == hipSuccess ? FT_OK : FT_ERR_LAUNCH;
+}
+
+int launch_stage2(const Stage2Args& a, int d, int dtype, hipStream_t stream) {
+#define FT_DISPATCH_D(E)                                       \
+  switch (d) {                                                 \
+    case 32: return launch_stage2_inst<E, 32>(a, stream);      \
+    case 64: return launch_stage2_inst<E, 64>(a, stream);      \
+    case 128: return launch_stage2_inst<E, 128>(a, stream);    \
+    case 256: return launch_stage2_inst<E, 256>(a, stream);    \
+    default: return FT_ERR_HEAD_DIM;                           \
+  }
+  if (dtype == FT_DTYPE_F16) { FT_DISPATCH_D(F16) }
+  if (dtype == FT_DTYPE_BF16) { FT_DISPATCH_D(BF16) }
+#undef FT_DISPATCH_D
+  return FT_ERR_DTYPE;
+}
+
+int check_common(int d, int g, int dtype) {
+  if (dtype != FT_DTYPE_F16 && dtype != FT_DTYPE_BF16) return FT_ERR_DTYPE;
+  if (d != 32 && d != 64 && d != 128 && d != 256) return FT_ERR_HEAD_DIM;
+  if (g < 1 || g > 64) return FT_ERR_GROUP;
+  return FT_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* ft_version(void) { return "fasttree_hip 0.1 (gfx950)"; }
+
+const char* ft_error_string(int code) {
+  switch (code) {
+    case FT_OK: return "ok";
+    case FT_ERR_NULL_POINTER: return "null pointer argument";
+    case FT_ERR_DTYPE: return "unsupported dtype (fp16 and bf16 only)";
+    case FT_ERR_HEAD_DIM: return "unsupported head dimension (32, 64, 128, 256)";
+    case FT_ERR_GROUP: return "unsupported query/KV head ratio";
+    case FT_ERR_ALIGNMENT: return "pointer or stride not aligned as required";
+    case FT_ERR_ARGUMENT: return "argument out of range";
+    case FT_ERR_LAUNCH: return "kernel launch failed";
+    default: return "unknown error";
+  }
+}
+
+int ft_stage1(const void* q, const void* k, const void* v,
+              int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+              const int32_t* vnode_to_kv_entries, const int32_t* vnode_to_kv_offs,
+              const int32_t* vnode_to_kv_lens, const int32_t* vnode_to_q_entries,
+              const int32_t* vnode_to_q_offs, const int32_t* vnode_to_q_lens,
+              int vnode_begin, int vnode_count, int num_kv_heads, int kv_group_num, int head_dim,
+              int q_tile, int kv_tile, float sm_scale,
+              float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
+              int dtype, ft_stream_t stream) {
+  (void)kv_tile;
+  if (int rc = check_common(head_dim, kv_group_num, dtype)) return rc;
+  if (vnode_count == 0) return FT_OK;
+  if (!q || !k || !v || !vnode_to_kv_entries || !vnode_to_kv_offs || !vnode_to_kv_lens || !vnode_to_q_entries ||
+      !vnode_to_q_offs || !vnode_to_q_lens || !mid_o || !mid_lse)
+    return FT_ERR_NULL_POINTER;
+  if (vnode_begin < 0 || vnode_count < 0 || num_kv_heads < 1 || num_kv_heads > 65535 || q_tile < 1 || !(sm_scale > 0.f))
+    return FT_ERR_ARGUMENT;
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(mid_o) || (sq0 | sq1 | sk0 | sk1 | sv0 | sv1) % 8 != 0 ||
+      (so0 | so1) % 4 != 0)
+    return FT_ERR_ALIGNMENT;
+  Stage1Args a{};
+  a.q = static_cast<const char*>(q);
+  a.k = static_cast<const char*>(k);
+  a.v = static_cast<const char*>(v);
+  a.sq0 = sq0; a.sq1 = sq1; a.sk0 = sk0; a.sk1 = sk1; a.sv0 = sv0; a.sv1 = sv1;
+  a.kv_entries = vnode_to_kv_entries; a.kv_offs = vnode_to_kv_offs; a.kv_lens = vnode_to_kv_lens;
+  a.q_entries = vnode_to_q_entries; a.q_offs = vnode_to_q_offs; a.q_lens = vnode_to_q_lens;
+  a.vnode_begin = vnode_begin; a.vnode_count = vnode_count;
+  a.g = kv_group_num;
+  a.scale_log2 = sm_scale * kLog2e;
+  a.mid_o = mid_o; a.so0 = so0; a.so1 = so1; a.mid_lse = mid_lse; a.sl0 = sl0;
+  const int64_t rows = (int64_t)q_tile * kv_group_num;
+  return launch_stage1<false>(a, num_kv_heads, head_dim, rows > 64 ? 64 : (int)rows, dtype, stream);
+}
+
+int ft_stage2(const int32_t* req_to_vnode_entries, const int32_t* req_to_vnode_offs,
+              const int32_t* req_to_vnode_lens,
+              const float* mid_o, int64_t so0, int64_t so1, const float* mid_lse, int64_t sl0,
+              void* o, int64_t oo0, int64_t oo1,
+              int batch_size, int num_qo_heads, int head_dim, int dtype, ft_stream_t stream) {
+  if (int rc = check_common(head_dim, 1, dtype)) return rc;
+  if (batch_size == 0) return FT_OK;
+  if (!req_to_vnode_entries || !req_to_vnode_offs || !req_to_vnode_lens || !mid_o || !mid_lse || !o)
+    return FT_ERR_NULL_POINTER;
+  if (batch_size < 0 || num_qo_heads < 1) return FT_ERR_ARGUMENT;
+  if (!aligned16(mid_o) || !aligned16(o) || (so0 | so1) % 4 != 0 || (oo0 | oo1) % 4 != 0) return FT_ERR_ALIGNMENT;
+  Stage2Args a{};
+  a.req_entries = req_to_vnode_entries; a.req_offs = req_to_vnode_offs; a.req_lens = req_to_vnode_lens;
+  a.mid_o = mid_o; a.so0 = so0; a.so1 = so1; a.mid_lse = mid_lse; a.sl0 = sl0;
+  a.o = static_cast<char*>(o); a.oo0 = oo0; a.oo1 = oo1;
+  a.batch = batch_size; a.hq = num_qo_heads; a.nsplit = 0;
+  return launch_stage2(a, head_dim, dtype, stream);
+}
+
+int ft_decode(const void* q, const void* k, const void* v, void* o,
+              int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+              int64_t oo0, int64_t oo1,
+              const int32_t* vnode_to_kv_entries, const int32_t* vnode_to_kv_offs,
+              const int32_t* vnode_to_kv_lens, const int32_t* vnode_to_q_entries,
+              const int32_t* vnode_to_q_offs, const int32_t* vnode_to_q_lens,
+              const int32_t* req_to_vnode_entries, const int32_t* req_to_vnode_offs,
+              const int32_t* req_to_vnode_lens,
+              float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
+              const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
+              const int32_t phase_q_tile_sizes[2], const int32_t phase_kv_tile_sizes[2],
+              int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
+              float sm_scale, int dtype, ft_stream_t stream) {
+  if (!phase_node_nums || !phase_node_offsets || !phase_q_tile_sizes || !phase_kv_tile_sizes) return FT_ERR_NULL_POINTER;
+  if (num_kv_heads < 1 || num_qo_heads % num_kv_heads != 0) return FT_ERR_GROUP;
+  const int g = num_qo_heads / num_kv_heads;
+  for (int phase = 0; phase < 2; ++phase) {
+    if (phase_node_nums[phase] == 0) continue;
+    if (int rc = ft_stage1(q, k, v, sq0, sq1, sk0, sk1, sv0, sv1, vnode_to_kv_entries, vnode_to_kv_offs,
+                           vnode_to_kv_lens, vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens,
+                           phase_node_offsets[phase], phase_node_nums[phase], num_kv_heads, g, head_dim,
+                           phase_q_tile_sizes[phase], phase_kv_tile_sizes[phase], sm_scale, mid_o, so0, so1,
+                           mid_lse, sl0, dtype, stream))
+      return rc;
+  }
+  return ft_stage2(req_to_vnode_entries, req_to_vnode_offs, req_to_vnode_lens, mid_o, so0, so1, mid_lse, sl0, o, oo0,
+                   oo1, batch_size, num_qo_heads, head_dim, dtype, stream);
+}
+
+int ft_gathered_decode(const void* q, const void* k_cache, const void* v_cache,
+                       const int32_t* cache_seqlens, void* o,
+                       int64_t sq0, int64_t sq1, int64_t oo0, int64_t oo1,
+                       int batch_size, int max_seqlen, int num_qo_heads, int num_kv_heads,
+                       int head_dim, int kv_split, float sm_scale,
+                       float* mid_o, float* mid_lse, int dtype, ft_stream_t stream) {
+  if (num_kv_heads < 1 || num_qo_heads % num_kv_heads != 0) return FT_ERR_GROUP;
+  const int g = num_qo_heads / num_kv_heads;
+  if (int rc = check_common(head_dim, g, dtype)) return rc;
+  if (batch_size == 0) return FT_OK;
+  if (!q || !k_cache || !v_cache || !cache_seqlens || !o || !mid_o || !mid_lse) return FT_ERR_NULL_POINTER;
+  if (batch_size < 0 || max_seqlen < 1 || kv_split < 1 || num_kv_heads > 65535 || !(sm_scale > 0.f)) return FT_ERR_ARGUMENT;
+  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(mid_o) || !aligned16(o) ||
+      (sq0 | sq1) % 8 != 0 || (oo0 | oo1) % 4 != 0)
+    return FT_ERR_ALIGNMENT;
+  const int nsplit = (max_seqlen + kv_split - 1) / kv_split;
+  if ((int64_t)batch_size * nsplit > INT32_MAX) return FT_ERR_ARGUMENT;
+  Stage1Args a{};
+  a.q = static_cast<const char*>(q);
+  a.k = static_cast<const char*>(k_cache);
+  a.v = static_cast<const char*>(v_cache);
+  a.sq0 = sq0; a.sq1 = sq1;
+  a.sk0 = a.sv0 = (int64_t)num_kv_heads * head_dim;
+  a.sk1 = a.sv1 = head_dim;
+  a.vnode_begin = 0; a.vnode_count = batch_size * nsplit;
+  a.g = g;
+  a.scale_log2 = sm_scale * kLog2e;
+  a.mid_o = mid_o; a.so0 = (int64_t)num_qo_heads * head_dim; a.so1 = head_dim;
+  a.mid_lse = mid_lse; a.sl0 = num_qo_heads;
+  a.cache_seqlens = cache_seqlens; a.max_seqlen = max_seqlen; a.kv_split = kv_split; a.nsplit = nsplit;
+  if (int rc = launch_stage1<true>(a, num_kv_heads, head_dim, g > 64 ? 64 : g, dtype, stream)) return rc;
+  Stage2Args b{};
+  b.mid_o = mid_o; b.so0 = a.so0; b.so1 = a.so1; b.mid_lse = mid_lse; b.sl0 = a.sl0;
+  b.o = static_cast<char*>(o); b.oo0 = oo0; b.oo1 = oo1;
+  b.batch = batch_size; b.hq = num_qo_heads; b.nsplit = nsplit;
+  return launch_stage2(b, head_dim, dtype, stream);
+}
+
+}  // extern "C"

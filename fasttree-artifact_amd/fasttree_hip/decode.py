@@ -1,0 +1,143 @@
+"""Python entry points of the decode path: thin argument marshalling over the C ABI.
+
+``fasttree_decode`` keeps the reference's positional signature
+(kernel_bench/fasttree.py:582-604; called positionally at kernel_bench/benchmark.py:115-124
+and with ``sm_scale=`` / ``logit_cap=`` keywords by the SGLang plugin, plugin.py:28-50).
+Work is enqueued on torch's current stream; nothing is synchronised or allocated.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+_DTYPES = {torch.float16: _lib.FT_DTYPE_F16, torch.bfloat16: _lib.FT_DTYPE_BF16}
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise _lib.FastTreeLibraryError(f"unsupported dtype {t.dtype}: fp16 and bf16 only") from None
+
+
+def _stream_handle(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _need_gpu(*tensors):
+    for t in tensors:
+        if not t.is_cuda:
+            raise _lib.FastTreeLibraryError("fasttree_decode needs device tensors; there is no CPU path")
+
+
+def _need_i32(*tensors):
+    for t in tensors:
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise _lib.FastTreeLibraryError("index tensors must be contiguous int32")
+
+
+def _need_inner_contiguous(*tensors):
+    for t in tensors:
+        if t.stride(-1) != 1:
+            raise _lib.FastTreeLibraryError("the last dimension of q, k, v, o and the scratch must be contiguous")
+
+
+def fasttree_decode(
+    q, k_buffer, v_buffer, o,
+    vnode_to_kv_entries, vnode_to_kv_offs, vnode_to_kv_lens,
+    vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens,
+    req_to_vnode_entries, req_to_vnode_offs, req_to_vnode_lens,
+    mid_o, mid_lse,
+    phase_node_nums, phase_node_offsets, phase_q_tile_sizes, phase_kv_tile_sizes,
+    sm_scale, logit_cap=-1,
+):
+    """Tree-structured decode attention; the result is written into ``o``.
+
+    ``logit_cap`` is accepted and ignored, as in the reference (fasttree.py:603).
+    """
+    assert q.shape[-1] == k_buffer.shape[-1]          # fasttree.py:437-438
+    _need_gpu(q, k_buffer, v_buffer, o, mid_o, mid_lse, vnode_to_kv_entries)
+    _need_inner_contiguous(q, k_buffer, v_buffer, o, mid_o, mid_lse)
+    _need_i32(vnode_to_kv_entries, vnode_to_kv_offs, vnode_to_kv_lens, vnode_to_q_entries, vnode_to_q_offs,
+              vnode_to_q_lens, req_to_vnode_entries, req_to_vnode_offs, req_to_vnode_lens)
+    if k_buffer.dtype != q.dtype or v_buffer.dtype != q.dtype or o.dtype != q.dtype:
+        raise _lib.FastTreeLibraryError("q, k, v and o must share one dtype")
+    if mid_o.dtype != torch.float32 or mid_lse.dtype != torch.float32:
+        raise _lib.FastTreeLibraryError("mid_o and mid_lse must be float32")
+    lib = _lib.load()
+    rc = lib.ft_decode(
+        q.data_ptr(), k_buffer.data_ptr(), v_buffer.data_ptr(), o.data_ptr(),
+        q.stride(0), q.stride(1), k_buffer.stride(0), k_buffer.stride(1),
+        v_buffer.stride(0), v_buffer.stride(1), o.stride(0), o.stride(1),
+        vnode_to_kv_entries.data_ptr(), vnode_to_kv_offs.data_ptr(), vnode_to_kv_lens.data_ptr(),
+        vnode_to_q_entries.data_ptr(), vnode_to_q_offs.data_ptr(), vnode_to_q_lens.data_ptr(),
+        req_to_vnode_entries.data_ptr(), req_to_vnode_offs.data_ptr(), req_to_vnode_lens.data_ptr(),
+        mid_o.data_ptr(), mid_o.stride(0), mid_o.stride(1), mid_lse.data_ptr(), mid_lse.stride(0),
+        _lib.int32_pair(phase_node_nums), _lib.int32_pair(phase_node_offsets),
+        _lib.int32_pair(phase_q_tile_sizes), _lib.int32_pair(phase_kv_tile_sizes),
+        q.shape[0], q.shape[1], k_buffer.shape[1], q.shape[-1],
+        float(sm_scale), _dtype_code(q), _stream_handle(q),
+    )
+    _lib.check(rc, "ft_decode")
+
+
+def fasttree_decode_stage1(q, k_buffer, v_buffer, vnode_to_kv_entries, vnode_to_kv_offs, vnode_to_kv_lens,
+                           vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, sm_scale, mid_o, mid_lse,
+                           phase_node_nums, phase_node_offsets, phase_q_tile_sizes, phase_kv_tile_sizes):
+    """Stage 1 alone (both phases): fills ``mid_o`` / ``mid_lse``
+    (the role of _fasttree_decode_stage1, kernel_bench/fasttree.py:416-479)."""
+    _need_gpu(q, k_buffer, v_buffer, mid_o, mid_lse)
+    lib = _lib.load()
+    hq, hkv = q.shape[1], k_buffer.shape[1]
+    for num, off, qt, kt in zip(phase_node_nums, phase_node_offsets, phase_q_tile_sizes, phase_kv_tile_sizes):
+        if num == 0:
+            continue
+        rc = lib.ft_stage1(
+            q.data_ptr(), k_buffer.data_ptr(), v_buffer.data_ptr(),
+            q.stride(0), q.stride(1), k_buffer.stride(0), k_buffer.stride(1), v_buffer.stride(0), v_buffer.stride(1),
+            vnode_to_kv_entries.data_ptr(), vnode_to_kv_offs.data_ptr(), vnode_to_kv_lens.data_ptr(),
+            vnode_to_q_entries.data_ptr(), vnode_to_q_offs.data_ptr(), vnode_to_q_lens.data_ptr(),
+            int(off), int(num), hkv, hq // hkv, q.shape[-1], int(qt), int(kt), float(sm_scale),
+            mid_o.data_ptr(), mid_o.stride(0), mid_o.stride(1), mid_lse.data_ptr(), mid_lse.stride(0),
+            _dtype_code(q), _stream_handle(q),
+        )
+        _lib.check(rc, "ft_stage1")
+
+
+def fasttree_decode_stage2(req_to_vnode_entries, req_to_vnode_offs, req_to_vnode_lens, mid_o, mid_lse, o):
+    """Stage 2 alone (the role of _fasttree_decode_stage2, kernel_bench/fasttree.py:549-579)."""
+    _need_gpu(mid_o, mid_lse, o)
+    lib = _lib.load()
+    rc = lib.ft_stage2(
+        req_to_vnode_entries.data_ptr(), req_to_vnode_offs.data_ptr(), req_to_vnode_lens.data_ptr(),
+        mid_o.data_ptr(), mid_o.stride(0), mid_o.stride(1), mid_lse.data_ptr(), mid_lse.stride(0),
+        o.data_ptr(), o.stride(0), o.stride(1), o.shape[0], o.shape[1], o.shape[2],
+        _dtype_code(o), _stream_handle(o),
+    )
+    _lib.check(rc, "ft_stage2")
+
+
+def gathered_decode(q, k_cache, v_cache, cache_seqlens, o, sm_scale, kv_split=512, mid_o=None, mid_lse=None):
+    """Decode attention without prefix sharing over a per-request gathered cache
+    ``[B, max_seqlen, Hkv, D]`` -- the baseline the tree path is compared with (the layout
+    of kernel_bench/flash_attn_wrap.py:36-70).  Scratch is allocated when not passed."""
+    _need_gpu(q, k_cache, v_cache, cache_seqlens, o)
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise _lib.FastTreeLibraryError("k_cache and v_cache must be contiguous")
+    batch, width, hkv, d = k_cache.shape
+    nsplit = (width + kv_split - 1) // kv_split
+    hq = q.shape[1]
+    if mid_o is None:
+        mid_o = torch.empty((batch * nsplit, hq, d), dtype=torch.float32, device=q.device)
+        mid_lse = torch.empty((batch * nsplit, hq), dtype=torch.float32, device=q.device)
+    lib = _lib.load()
+    rc = lib.ft_gathered_decode(
+        q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), cache_seqlens.data_ptr(), o.data_ptr(),
+        q.stride(0), q.stride(1), o.stride(0), o.stride(1),
+        batch, width, hq, hkv, d, int(kv_split), float(sm_scale),
+        mid_o.data_ptr(), mid_lse.data_ptr(), _dtype_code(q), _stream_handle(q),
+    )
+    _lib.check(rc, "ft_gathered_decode")
+    return mid_o, mid_lse

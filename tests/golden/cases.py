@@ -149,14 +149,14 @@ PLANNER_CASES = _planner_cases()
 def _kernel_cases():
     """Small enough for Triton's CPU interpreter to finish in minutes.  TSQs are chosen so
     the planner's adaptation leaves them unchanged (the bench hands its original tile
-    lists to the kernel, kernel_bench/benchmark.py:121-122)."""
+    lists to the kernel, kernel_bench/benchmark.py:121-122).  All cases are fp16: the
+    interpreter has no bfloat16 arithmetic (it computes on the raw bit patterns), so bf16
+    is checked against the dense fp64 identity instead."""
     big = dict(para_threshs1=(1, 1), para_threshs2=(1, 1))  # never adapt
     return [
         _case("k_kat1_mha", regular([1, 1, 2], [100, 50, 10]), 4, 4, D=64, dtype="fp16", seed=11, **big),
         _case("k_two_level_gqa4", regular([1, 6], [200, 37]), 8, 2, D=128, dtype="fp16", seed=12, **big),
         _case("k_three_level_gqa4", regular([1, 3, 24], [150, 70, 19]), 8, 2, D=128, dtype="fp16", seed=13,
-              kv_split_sizes=(64, 32), **big),
-        _case("k_three_level_bf16", regular([1, 3, 24], [150, 70, 19]), 8, 2, D=128, dtype="bf16", seed=14,
               kv_split_sizes=(64, 32), **big),
         _case("k_irregular_gqa8", irregular(5, levels=4, fanout_range=(1, 4), len_range=(4, 90), max_leaves=40),
               16, 2, D=128, dtype="fp16", seed=15, kv_split_sizes=(128, 32), **big),

@@ -1,0 +1,328 @@
+"""Parity of the HIP decode path, called through the C ABI, on a real MI355X.
+
+Bar (per request): max-abs <= 2e-3 and mean-abs <= 1e-3 against the reference kernels'
+own outputs where fixtures hold them, else against the fp64 dense oracle (for bf16 the
+oracle is rounded to bf16 first: bf16 carries 8 significant bits, so the comparison is
+made on the rounding grid the output lives on and the same bar applies to fp32 partials).
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import fasttree_oracle as oracle
+from cases import KERNEL_CASES, PLANNER_CASES, build_tree, kernel_case_inputs
+from fasttree_hip.decode import (fasttree_decode, fasttree_decode_stage1, fasttree_decode_stage2,
+                                 gathered_decode)
+from fasttree_hip.inputs import gather_per_request, make_decode_inputs, request_paths
+from fasttree_hip.planner import FastTreeParams, fasttree_plan, fasttree_preparation
+from helpers import (MAX_ABS_TOL, MEAN_ABS_TOL, assert_parity, bits16_to_tensor, kernel_golden, per_request_errors,
+                     plan_to_device, run_planner)
+
+pytestmark = pytest.mark.gpu
+
+
+def _announce(*what):
+    print("\n[gpu case]", *what, flush=True)
+
+
+def _decode(q, k, v, aux, q_tiles, kv_tiles, scale):
+    o = torch.full_like(q, float("nan"))
+    fasttree_decode(q, k, v, o, *aux, q_tiles, kv_tiles, scale)
+    torch.cuda.synchronize()
+    return o
+
+
+@pytest.mark.parametrize("shuffled", [False, True], ids=["node_major_pool", "shuffled_pool"])
+@pytest.mark.parametrize("case", KERNEL_CASES, ids=[c["name"] for c in KERNEL_CASES])
+def test_matches_reference_kernel_outputs(case, shuffled, device):
+    """Same tree, same Q/K/V bits, same plan as the fixture: o, mid_o and mid_lse agree with
+    what the reference's kernels wrote."""
+    _announce(case["name"], "shuffled" if shuffled else "node-major")
+    tree, ptrs, batch = build_tree(case["tree"])
+    q, k, v = kernel_case_inputs(case, tree, ptrs, batch)
+    slot_map = np.random.default_rng(99).permutation(ptrs[-1]) if shuffled else None
+    _, _, _, plan, params, _ = run_planner(case, kv_slot_map=slot_map)
+    if shuffled:
+        where = torch.from_numpy(slot_map)
+        k_pool, v_pool = torch.empty_like(k), torch.empty_like(v)
+        k_pool[where], v_pool[where] = k, v
+    else:
+        k_pool, v_pool = k, v
+    aux = plan_to_device(plan, case["Hq"], case["D"], device)
+    gold = kernel_golden(case["name"])
+    o = _decode(q.to(device), k_pool.to(device), v_pool.to(device), aux, case["TSQs"], case["TSKs"],
+                1.0 / math.sqrt(case["D"]))
+    assert_parity(o, bits16_to_tensor(gold["o"], torch.float16), case["name"])
+    assert_parity(aux[9], torch.from_numpy(gold["mid_o"]), case["name"] + " mid_o")
+    lse_err = (aux[10].cpu() - torch.from_numpy(gold["mid_lse"])).abs().max()
+    assert lse_err <= 1e-3, f"mid_lse {lse_err}"
+
+
+def _dense_check(tree, inp, o, what, sample=None, dtype=torch.float16):
+    reqs = list(range(inp.batch_size)) if sample is None else sample
+    paths = [inp.path_tokens[r] for r in reqs]
+    q_cpu, k_cpu, v_cpu = inp.Q.cpu(), inp.K_pool.cpu(), inp.V_pool.cpu()
+    dense = oracle.dense_attention(q_cpu[reqs], k_cpu, v_cpu, paths, 1.0 / math.sqrt(q_cpu.shape[-1]))
+    return assert_parity(o[reqs], dense.to(dtype), what)
+
+
+CONFIGS = {
+    # name: (sizes, lens, Hq, Hkv, dtype, seed)
+    "c1": ([1, 16], [1024, 128], 32, 32, torch.float16, 1),
+    "c2": ([1, 64], [4096, 256], 32, 8, torch.float16, 2),
+    "c3": ([1, 10, 400], [4000, 400, 40], 32, 8, torch.float16, 3),
+}
+# (q tiles, kv split sizes, thresholds 1, thresholds 2): the reference bench's values and a
+# preset sized for 256 compute units with 64-request tiles
+PRESETS = {
+    "reference_defaults": (None, (1024, 128), (132, 528), (132, 132)),
+    "wide_tiles": ("wide", (1024, 128), (256, 1024), (256, 256)),
+}
+
+
+@pytest.mark.parametrize("preset", list(PRESETS))
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_baseline_configs_against_dense_oracle(name, preset, device):
+    """C1-C3 at full size, shuffled paged pool: every request against the fp64 oracle."""
+    _announce(name, preset)
+    sizes, lens, hq, hkv, dtype, seed = CONFIGS[name]
+    tree, ptrs, batch = build_tree({"kind": "regular", "sizes": sizes, "lens": lens})
+    inp = make_decode_inputs(tree, hq, hkv, 128, device=device, dtype=dtype, seed=seed, shuffle_slots=True)
+    g = hq // hkv
+    tiles, splits, thr1, thr2 = PRESETS[preset]
+    q_tiles = [max(1, 64 // g), max(1, 16 // g)] if tiles is None else [64, max(1, 16 // g)]
+    params = FastTreeParams()
+    params.set_values(0.66, 0.33, 0.1); params.set_q_tile_sizes(list(q_tiles)); params.set_kv_tile_sizes([32, 32])
+    params.set_kv_group_num(g)
+    aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, hq, hkv, 128, list(splits), list(thr1), list(thr2), params,
+                                  device=device, kv_slot_map=inp.slot_map)
+    o = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, q_tiles, [32, 32], 1.0 / math.sqrt(128))
+    sample = None if batch <= 64 else list(range(0, batch, 7))
+    print(_dense_check(tree, inp, o, f"{name}/{preset}", sample), flush=True)
+    # every request against an fp32 torch attention on the device (gathered per request)
+    k_cache, v_cache, lens_t = gather_per_request(inp)
+    mask = torch.arange(k_cache.shape[1], device=device)[None, :] < lens_t[:, None]
+    s = torch.einsum("bkgd,blkd->bkgl", inp.Q.float().view(batch, hkv, g, 128), k_cache.float()) / math.sqrt(128)
+    s = s.masked_fill(~mask[:, None, None, :], float("-inf"))
+    ref = torch.einsum("bkgl,blkd->bkgd", torch.softmax(s, dim=-1), v_cache.float().masked_fill(~mask[:, :, None, None], 0))
+    assert_parity(o, ref.reshape(batch, hq, 128), f"{name}/{preset} vs torch fp32")
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_deep_irregular_tree(seed, device):
+    """C5: 5 levels, fan-out U[1,8], lengths log-uniform [16,2048], <= 1024 leaves, GQA 8."""
+    _announce("c5", seed)
+    tree, ptrs, batch = build_tree({"kind": "irregular", "seed": seed})
+    inp = make_decode_inputs(tree, 64, 8, 128, device=device, dtype=torch.float16, seed=seed, shuffle_slots=True)
+    params = FastTreeParams()
+    params.set_q_tile_sizes([8, 2]); params.set_kv_tile_sizes([32, 32]); params.set_kv_group_num(8)
+    aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, 64, 8, 128, [1024, 128], [132, 528], [132, 132], params,
+                                  device=device, kv_slot_map=inp.slot_map)
+    o = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, list(params.TSQs), [32, 32], 1.0 / math.sqrt(128))
+    step = max(1, batch // 48)
+    print(_dense_check(tree, inp, o, f"c5 seed {seed}", list(range(0, batch, step))), flush=True)
+
+
+def test_wide_shallow_tree_bf16(device):
+    """C4: 512-token root, 2048 leaves of 1024 tokens, bf16, > 2^31 pool elements (needs
+    64-bit addressing).  Sampled requests against the fp64 oracle rounded to bf16."""
+    _announce("c4")
+    tree, ptrs, batch = build_tree({"kind": "regular", "sizes": [1, 2048], "lens": [512, 1024]})
+    inp = make_decode_inputs(tree, 32, 8, 128, device=device, dtype=torch.bfloat16, seed=4, shuffle_slots=True,
+                             host_rng=False)
+    assert inp.K_pool.numel() > 2 ** 31
+    params = FastTreeParams()
+    params.set_q_tile_sizes([16, 4]); params.set_kv_tile_sizes([32, 32]); params.set_kv_group_num(4)
+    aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, 32, 8, 128, [1024, 128], [132, 528], [132, 132], params,
+                                  device=device, kv_slot_map=inp.slot_map)
+    o = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, [16, 4], [32, 32], 1.0 / math.sqrt(128))
+    high = [r for r in range(batch) if int(inp.path_tokens[r].max()) * 8 * 128 >= 2 ** 31]
+    assert high, "some request must read pool rows beyond 2^31 elements"
+    sample = sorted(set([0, 1, 511, 1024, 2046, 2047] + high[:3]))
+    q_cpu = inp.Q[sample].cpu()
+    paths = [inp.path_tokens[r] for r in sample]
+    # gather only the sampled rows to the host (the pool is 4 GB)
+    uniq = np.unique(np.concatenate(paths))
+    remap = {int(s): i for i, s in enumerate(uniq)}
+    k_small = inp.K_pool[torch.from_numpy(uniq).to(device)].cpu()
+    v_small = inp.V_pool[torch.from_numpy(uniq).to(device)].cpu()
+    small_paths = [np.array([remap[int(s)] for s in p]) for p in paths]
+    dense = oracle.dense_attention(q_cpu, k_small, v_small, small_paths, 1.0 / math.sqrt(128))
+    # bf16 output: compare on the bf16 grid; partial sums are fp32 so the bar is unchanged
+    assert_parity(o[sample], dense.to(torch.bfloat16), "c4 sampled")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("d", [32, 64, 128, 256])
+@pytest.mark.parametrize("heads", [(4, 4), (8, 2), (16, 2), (16, 1)], ids=["mha", "gqa4", "gqa8", "gqa16"])
+def test_head_dims_groups_and_dtypes(heads, d, dtype, device):
+    _announce("shape sweep", heads, d, dtype)
+    hq, hkv = heads
+    g = hq // hkv
+    tree, ptrs, batch = build_tree({"kind": "irregular", "seed": 21, "levels": 4, "fanout_range": (1, 5),
+                                    "len_range": (1, 150), "max_leaves": 50})
+    inp = make_decode_inputs(tree, hq, hkv, d, device=device, dtype=dtype, seed=d + hq, shuffle_slots=True)
+    q_tiles = [max(1, 64 // g), max(1, 16 // g)]
+    params = FastTreeParams()
+    params.set_q_tile_sizes(list(q_tiles)); params.set_kv_tile_sizes([32, 32]); params.set_kv_group_num(g)
+    aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, hq, hkv, d, [256, 64], [132, 528], [132, 132], params,
+                                  device=device, kv_slot_map=inp.slot_map)
+    o = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, list(params.TSQs), list(params.TSKs), 1.0 / math.sqrt(d))
+    _dense_check(tree, inp, o, f"{heads} d={d} {dtype}", dtype=dtype)
+
+
+def test_stage_outputs_against_restated_arithmetic(device):
+    """mid_o is normalised by its own sum, mid_lse is a natural-log log-sum-exp; stage 2 alone
+    merges oracle partials."""
+    _announce("stage split")
+    case = next(c for c in KERNEL_CASES if c["name"] == "k_irregular_gqa8")
+    tree, ptrs, batch, plan, params, _ = run_planner(case)
+    q, k, v = kernel_case_inputs(case, tree, ptrs, batch)
+    scale = 1.0 / math.sqrt(case["D"])
+    o_ref, mid_o_ref, mid_lse_ref = oracle.fasttree_decode_arith(q, k, v, plan, 32, scale)
+    aux = plan_to_device(plan, case["Hq"], case["D"], device)
+    fasttree_decode_stage1(q.to(device), k.to(device), v.to(device), *aux[:6], scale, aux[9], aux[10],
+                           aux[11], aux[12], case["TSQs"], case["TSKs"])
+    torch.cuda.synchronize()
+    assert_parity(aux[9], mid_o_ref, "mid_o")
+    assert (aux[10].cpu() - mid_lse_ref).abs().max() <= 1e-3
+    o = torch.empty_like(q, device=device)
+    fasttree_decode_stage2(aux[6], aux[7], aux[8], mid_o_ref.to(device), mid_lse_ref.to(device), o)
+    torch.cuda.synchronize()
+    assert_parity(o, o_ref, "stage 2 on oracle partials")
+
+
+def test_strided_views_and_padded_scratch(device):
+    """q / o / pool rows taken as views of wider tensors, scratch larger than needed (as the
+    serving plugin pre-allocates it), and a 2-D index array used flat."""
+    _announce("strided views")
+    hq, hkv, d = 8, 2, 128
+    tree, ptrs, batch = build_tree({"kind": "regular", "sizes": [1, 3, 9], "lens": [70, 33, 5]})
+    inp = make_decode_inputs(tree, hq, hkv, d, device=device, dtype=torch.float16, seed=8, shuffle_slots=True)
+    params = FastTreeParams()
+    params.set_q_tile_sizes([16, 4]); params.set_kv_tile_sizes([32, 32]); params.set_kv_group_num(4)
+    aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, hq, hkv, d, [64, 32], [1, 1], [1, 1], params,
+                                  device=device, kv_slot_map=inp.slot_map)
+    wide_q = torch.zeros(batch, hq + 3, d + 64, dtype=torch.float16, device=device)
+    q_view = wide_q[:, 1:1 + hq, 32:32 + d]
+    q_view.copy_(inp.Q)
+    total = inp.K_pool.shape[0]
+    wide_k = torch.zeros(total, hkv * 2, d, dtype=torch.float16, device=device)
+    wide_v = torch.zeros(total, hkv * 2, d, dtype=torch.float16, device=device)
+    k_view, v_view = wide_k[:, ::2], wide_v[:, 1::2]
+    k_view.copy_(inp.K_pool); v_view.copy_(inp.V_pool)
+    wide_o = torch.zeros(batch, hq, 2 * d, dtype=torch.float16, device=device)
+    o_view = wide_o[..., d:]
+    rows = aux[3].numel()
+    big_mid_o = torch.full((rows + 100, hq, d), float("nan"), dtype=torch.float32, device=device)
+    big_mid_lse = torch.full((rows + 100, hq), float("nan"), dtype=torch.float32, device=device)
+    entries_2d = torch.cat([aux[0], aux[0].new_full((8 - aux[0].numel() % 8,), -1)]).view(-1, 8)
+    fasttree_decode(q_view, k_view, v_view, o_view, entries_2d, *aux[1:9], big_mid_o, big_mid_lse, aux[11], aux[12],
+                    [16, 4], [32, 32], sm_scale=1.0 / math.sqrt(d), logit_cap=30.0)
+    torch.cuda.synchronize()
+    _dense_check(tree, inp, o_view, "strided")
+    assert torch.isnan(big_mid_o[rows:]).all() and (wide_o[..., :d] == 0).all()
+
+
+def test_tile_arguments_smaller_than_the_plan(device):
+    """The bench hands its original tile lists to the kernel even when the planner widened
+    them (kernel_bench/benchmark.py:121-122); vnodes wider than the tile argument are still
+    computed in full here."""
+    _announce("tile mismatch")
+    case = next(c for c in PLANNER_CASES if c["name"] == "kat1")
+    tree, ptrs, batch, plan, params, _ = run_planner(case)
+    assert params.TSQs == [64, 64]
+    inp = make_decode_inputs(tree, 32, 32, 128, device=device, dtype=torch.float16, seed=6, shuffle_slots=False)
+    aux = plan_to_device(plan, 32, 128, device)
+    for tiles in ([64, 16], [64, 64], [1, 1]):
+        o = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, tiles, [32, 32], 1.0 / math.sqrt(128))
+        _dense_check(tree, inp, o, f"tiles {tiles}")
+
+
+def test_all_merge_ablation_equals_per_request_attention(device):
+    """alpha = beta = 0, gamma = 10, split 81920: one vnode per request over its whole path."""
+    _announce("ablation")
+    tree, ptrs, batch = build_tree({"kind": "regular", "sizes": [1, 4, 32], "lens": [300, 120, 33]})
+    inp = make_decode_inputs(tree, 32, 8, 128, device=device, dtype=torch.float16, seed=9, shuffle_slots=True)
+    params = FastTreeParams()
+    params.set_values(0.0, 0.0, 10.0); params.set_q_tile_sizes([16, 4]); params.set_kv_tile_sizes([32, 32])
+    params.set_kv_group_num(4)
+    aux, assign = fasttree_preparation(tree, inp.KV_ptrs, batch, 32, 8, 128, [81920, 81920], [1, 1], [1, 1], params,
+                                       device=device, kv_slot_map=inp.slot_map)
+    assert all(a == 1 for a in assign[1:]) and aux[11] == [0, batch]
+    o = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, [16, 4], [32, 32], 1.0 / math.sqrt(128))
+    _dense_check(tree, inp, o, "all-merge")
+
+
+def test_single_token_and_single_node_trees(device):
+    _announce("tiny trees")
+    for rows in ([[-1, 0, 1, 0]], [[-1, 0, 1, 2], [0, 1, 1, 0], [0, 2, 1, 0]], [[-1, 0, 33, 0]]):
+        tree, ptrs, batch = build_tree({"kind": "rows", "rows": rows})
+        inp = make_decode_inputs(tree, 8, 2, 64, device=device, dtype=torch.float16, seed=1, shuffle_slots=True)
+        params = FastTreeParams()
+        params.set_q_tile_sizes([16, 4]); params.set_kv_tile_sizes([32, 32]); params.set_kv_group_num(4)
+        aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, 8, 2, 64, [1024, 128], [132, 528], [132, 132], params,
+                                      device=device, kv_slot_map=inp.slot_map)
+        o = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, list(params.TSQs), [32, 32], 0.125)
+        _dense_check(tree, inp, o, f"rows {rows}")
+
+
+def test_is_linear_in_v_and_repeatable(device):
+    """Size-independent properties at C2's full size: bit-identical on repeat; linear in V."""
+    _announce("c2 properties")
+    sizes, lens, hq, hkv, dtype, seed = CONFIGS["c2"]
+    tree, ptrs, batch = build_tree({"kind": "regular", "sizes": sizes, "lens": lens})
+    inp = make_decode_inputs(tree, hq, hkv, 128, device=device, dtype=dtype, seed=seed, shuffle_slots=True)
+    params = FastTreeParams()
+    params.set_q_tile_sizes([16, 4]); params.set_kv_tile_sizes([32, 32]); params.set_kv_group_num(4)
+    aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, hq, hkv, 128, [1024, 128], [132, 528], [132, 132], params,
+                                  device=device, kv_slot_map=inp.slot_map)
+    run = lambda v: _decode(inp.Q, inp.K_pool, v, aux, [16, 4], [32, 32], 1.0 / math.sqrt(128))
+    a, b = run(inp.V_pool), run(inp.V_pool)
+    assert torch.equal(a, b)
+    doubled = run(inp.V_pool * 2)          # exact in fp16: a power of two
+    assert torch.equal(doubled, a * 2)
+    ones = run(torch.ones_like(inp.V_pool))
+    assert (ones.float() - 1).abs().max() <= 1e-3      # soft-max weights sum to one
+
+
+@pytest.mark.parametrize("kv_split", [64, 512, 4096])
+def test_gathered_baseline(kv_split, device):
+    """The no-sharing baseline over the per-request gathered cache gives the same answers."""
+    _announce("gathered", kv_split)
+    tree, ptrs, batch = build_tree({"kind": "regular", "sizes": [1, 5, 20], "lens": [700, 90, 17]})
+    for hq, hkv in ((32, 8), (8, 8)):
+        inp = make_decode_inputs(tree, hq, hkv, 128, device=device, dtype=torch.float16, seed=3, shuffle_slots=True)
+        k_cache, v_cache, lens = gather_per_request(inp, max_seqlen=900)
+        o = torch.full_like(inp.Q, float("nan"))
+        gathered_decode(inp.Q, k_cache, v_cache, lens, o, 1.0 / math.sqrt(128), kv_split=kv_split)
+        torch.cuda.synchronize()
+        _dense_check(tree, inp, o, f"gathered {hq}/{hkv} split {kv_split}")
+
+
+def test_runs_on_a_side_stream_and_unsupported_inputs_raise(device):
+    _announce("stream / errors")
+    from fasttree_hip import _lib
+    tree, ptrs, batch = build_tree({"kind": "regular", "sizes": [1, 4], "lens": [50, 9]})
+    inp = make_decode_inputs(tree, 8, 2, 128, device=device, dtype=torch.float16, seed=2, shuffle_slots=True)
+    params = FastTreeParams()
+    params.set_q_tile_sizes([16, 4]); params.set_kv_tile_sizes([32, 32]); params.set_kv_group_num(4)
+    aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, 8, 2, 128, [1024, 128], [1, 1], [1, 1], params,
+                                  device=device, kv_slot_map=inp.slot_map)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    o = torch.full_like(inp.Q, float("nan"))
+    with torch.cuda.stream(side):
+        fasttree_decode(inp.Q, inp.K_pool, inp.V_pool, o, *aux, [16, 4], [32, 32], 1.0 / math.sqrt(128))
+    side.synchronize()
+    _dense_check(tree, inp, o, "side stream")
+    with pytest.raises(_lib.FastTreeLibraryError):
+        fasttree_decode(inp.Q.float(), inp.K_pool.float(), inp.V_pool.float(), o.float(), *aux, [16, 4], [32, 32], 0.1)
+    with pytest.raises(_lib.FastTreeLibraryError):
+        fasttree_decode(inp.Q, inp.K_pool, inp.V_pool, o, aux[0].long(), *aux[1:], [16, 4], [32, 32], 0.1)
+    bad = torch.zeros(batch, 8, 48, dtype=torch.float16, device=device)
+    with pytest.raises(AssertionError):
+        fasttree_decode(bad, bad, bad, bad, *aux, [16, 4], [32, 32], 0.1)
