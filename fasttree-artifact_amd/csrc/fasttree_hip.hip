@@ -61,24 +61,29 @@ struct BF16 {
   }
 };
 
-// Wave-wide exchange helpers.  v_permlane{16,32}_swap with both operands equal to x
-// return (x of the lower half, x of the upper half) of each 32-lane / 64-lane group.
-__device__ __forceinline__ float xor16_max(float x) {
-  auto r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, x), false, false);
-  return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+// Wave-wide exchange helpers.  v_permlane{16,32}_swap exchanges the odd 16-lane rows
+// (upper 32-lane half) of its first operand with the even rows (lower half) of its second;
+// fed the same value twice it yields (value of the even row / lower half, value of the odd
+// row / upper half) in every lane.  The two results are copied into scalars before they are
+// reinterpreted: a bit cast applied directly to an element of the returned vector reads
+// element 0 for both.
+struct LanePair { float lo, hi; };
+__device__ __forceinline__ LanePair halves16(float x) {
+  const unsigned a = __builtin_bit_cast(unsigned, x);
+  auto r = __builtin_amdgcn_permlane16_swap(a, a, false, false);
+  const unsigned r0 = r[0], r1 = r[1];
+  return {__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1)};
 }
-__device__ __forceinline__ float xor32_max(float x) {
-  auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, x), false, false);
-  return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+__device__ __forceinline__ LanePair halves32(float x) {
+  const unsigned a = __builtin_bit_cast(unsigned, x);
+  auto r = __builtin_amdgcn_permlane32_swap(a, a, false, false);
+  const unsigned r0 = r[0], r1 = r[1];
+  return {__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1)};
 }
-__device__ __forceinline__ float xor16_sum(float x) {
-  auto r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, x), false, false);
-  return __builtin_bit_cast(float, r[0]) + __builtin_bit_cast(float, r[1]);
-}
-__device__ __forceinline__ float xor32_sum(float x) {
-  auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, x), false, false);
-  return __builtin_bit_cast(float, r[0]) + __builtin_bit_cast(float, r[1]);
-}
+__device__ __forceinline__ float xor16_max(float x) { LanePair h = halves16(x); return fmaxf(h.lo, h.hi); }
+__device__ __forceinline__ float xor32_max(float x) { LanePair h = halves32(x); return fmaxf(h.lo, h.hi); }
+__device__ __forceinline__ float xor16_sum(float x) { LanePair h = halves16(x); return h.lo + h.hi; }
+__device__ __forceinline__ float xor32_sum(float x) { LanePair h = halves32(x); return h.lo + h.hi; }
 // Orders this wave's LDS traffic around a point where lanes read what other lanes of the
 // same wave wrote.  LDS executes one wave's instructions in order, so no wait is needed;
 // the fences only stop the compiler from moving accesses across.
