@@ -104,6 +104,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="c3", choices=list(WORKLOADS))
     ap.add_argument("--preset", default="mi355x", choices=list(PRESETS))
+    ap.add_argument("--q-tiles", default=None, help="override the preset's query tile sizes, e.g. 64,4")
+    ap.add_argument("--kv-splits", default=None, help="override the preset's KV split sizes, e.g. 1024,128")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gathered", action="store_true")
     ap.add_argument("--profile-only", action="store_true",
@@ -122,6 +124,14 @@ def main():
 
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.q_tiles or args.kv_splits:
+        custom = dict(PRESETS[args.preset])
+        if args.q_tiles:
+            custom["q_tiles"] = tuple(int(x) for x in args.q_tiles.split(","))
+        if args.kv_splits:
+            custom["kv_splits"] = tuple(int(x) for x in args.kv_splits.split(","))
+        PRESETS["custom"] = custom
+        args.preset = "custom"
     prob = build_problem(args.workload, args.preset, device)
     inp, aux = prob["inp"], prob["aux"]
     scale = 1.0 / math.sqrt(128)

@@ -25,6 +25,7 @@ namespace {
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
@@ -44,6 +45,9 @@ struct F16 {
   static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   }
+  static __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
   static __device__ __forceinline__ unsigned pack2(float lo, float hi) {
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
     h2 v = {(_Float16)lo, (_Float16)hi};
@@ -53,6 +57,9 @@ struct F16 {
 struct BF16 {
   static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   }
   static __device__ __forceinline__ unsigned pack2(float lo, float hi) {
     typedef __bf16 b2 __attribute__((ext_vector_type(2)));
@@ -170,19 +177,14 @@ template <int D, int NQB> struct WaveState {
   float l[NQB];  // running sum of this lane's own probabilities (reduced over lanes at the end)
 };
 
-// One wave attends NQB*16 query rows to tokens [tile0*32, ...) in steps of tile_step tiles.
-template <typename E, int D, int NQB, bool GATHERED>
-__device__ __forceinline__ void wave_attend(const Stage1Args& a, const VnodeView& vn, int kvh, int row0,
-                                            int tile0, int tile_step, char* lds, WaveState<D, NQB>& st) {
-  using G = TileGeom<D>;
-  constexpr int KS = D / 32, DB = D / 16;
+// Query fragments of one wave (B operand of S^T = K Q^T): qf[qb][ks] holds, for row
+// row0 + 16*qb + lane%16, the 8 dims 32*ks + 8*(lane/16) .. +7.  Rows past the vnode are zero.
+template <int D, int NQB, bool GATHERED>
+__device__ __forceinline__ void load_q_frags(const Stage1Args& a, const VnodeView& vn, int kvh, int row0,
+                                             u32x4 (&qf)[NQB][D / 32]) {
+  constexpr int KS = D / 32;
   const int lane = threadIdx.x & 63;
   const int p = lane & 15, c = lane >> 4;
-  char* ldsK = lds;
-  char* ldsV = lds + G::kBytesK;
-
-  // ---- query fragments (B operand of S^T = K Q^T): row 16*qb + p, dims 32*ks + 8*c .. +7
-  u32x4 qf[NQB][KS];
   const int rows_total = vn.q_len * a.g;
 #pragma unroll
   for (int qb = 0; qb < NQB; ++qb) {
@@ -198,14 +200,124 @@ __device__ __forceinline__ void wave_attend(const Stage1Args& a, const VnodeView
       qf[qb][ks] = ok ? *reinterpret_cast<const u32x4*>(src + 64 * ks) : z;
     }
   }
+}
 
+template <int D, int NQB>
+__device__ __forceinline__ void reset_state(WaveState<D, NQB>& st) {
 #pragma unroll
   for (int qb = 0; qb < NQB; ++qb) {
     st.m[qb] = -INFINITY;
     st.l[qb] = 0.f;
 #pragma unroll
-    for (int db = 0; db < DB; ++db) st.o[qb][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int db = 0; db < D / 16; ++db) st.o[qb][db] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
+}
+
+// every lane of a row gets the row's full probability sum
+template <int D, int NQB>
+__device__ __forceinline__ void finish_state(WaveState<D, NQB>& st) {
+#pragma unroll
+  for (int qb = 0; qb < NQB; ++qb) st.l[qb] = xor32_sum(xor16_sum(st.l[qb]));
+}
+
+// One 32-token step of a wave: scores of its NQB*16 rows against the tile staged at
+// (ldsK, ldsV), online soft-max update, P.V.  `valid` (>= 1) is how many of the 32 tokens exist.
+template <typename E, int D, int NQB>
+__device__ __forceinline__ void tile_step(const char* ldsK, const char* ldsV, int valid, float sc,
+                                          const u32x4 (&qf)[NQB][D / 32], WaveState<D, NQB>& st) {
+  using G = TileGeom<D>;
+  constexpr int KS = D / 32, DB = D / 16;
+  const int lane = threadIdx.x & 63;
+  const int p = lane & 15, c = lane >> 4;
+
+  // ---- S^T = K Q^T : s[tb][qb][j] = score(token 16*tb + 4*c + j, row 16*qb + p)
+  f32x4 s[2][NQB];
+#pragma unroll
+  for (int tb = 0; tb < 2; ++tb) {
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) s[tb][qb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const u32x4 kf = *reinterpret_cast<const u32x4*>(ldsK + (16 * tb + p) * G::kPitchK + 64 * ks + 16 * c);
+#pragma unroll
+      for (int qb = 0; qb < NQB; ++qb) s[tb][qb] = E::mfma(kf, qf[qb][ks], s[tb][qb]);
+    }
+  }
+
+  // tokens past the end of the run score -inf (wave-uniform branch: only a run's last tile)
+  if (valid < kTileTokens) {
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (16 * tb + 4 * c + j >= valid) {
+#pragma unroll
+          for (int qb = 0; qb < NQB; ++qb) s[tb][qb][j] = -INFINITY;
+        }
+  }
+
+  // Online soft-max with a lazily updated reference: a row's reference m only moves when the
+  // row's running maximum exceeds it by more than kSlack (log2 units), so probabilities stay
+  // below 2^kSlack -- exact in any case, since numerator and denominator share the reference --
+  // and the accumulators are rescaled rarely instead of on almost every tile.
+  constexpr float kSlack = 8.f;
+  u32x4 pf[NQB];
+#pragma unroll
+  for (int qb = 0; qb < NQB; ++qb) {
+    float mx = fmaxf(fmaxf(fmaxf(s[0][qb][0], s[0][qb][1]), fmaxf(s[0][qb][2], s[0][qb][3])),
+                     fmaxf(fmaxf(s[1][qb][0], s[1][qb][1]), fmaxf(s[1][qb][2], s[1][qb][3])));
+    mx = xor32_max(xor16_max(mx)) * sc;      // sc > 0; finite: the tile holds at least one token
+    const float m_old = st.m[qb];
+    const bool grow = mx > m_old + kSlack;   // also true on the first tile (m_old = -inf)
+    if (__builtin_amdgcn_ballot_w64(grow)) {
+      const float m_new = grow ? mx : m_old;
+      const float alpha = __builtin_amdgcn_exp2f(m_old - m_new);
+      st.l[qb] *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) st.o[qb][db] *= alpha;
+      st.m[qb] = m_new;
+    }
+    const float neg_m = -st.m[qb];
+    float x[8];
+    float sum = 0.f;
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        x[4 * tb + j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tb][qb][j], sc, neg_m));
+        sum += x[4 * tb + j];
+      }
+    st.l[qb] += sum;
+    pf[qb] = u32x4{E::pack2(x[0], x[1]), E::pack2(x[2], x[3]), E::pack2(x[4], x[5]), E::pack2(x[6], x[7])};
+  }
+
+  // ---- O^T += V^T P^T : A operand rows = dims 16*db + p, k slots = the 8 tokens this lane's P holds
+#pragma unroll
+  for (int db = 0; db < DB; ++db) {
+    const char* va = ldsV + (4 * c + (p >> 2)) * G::kPitchV + 2 * (16 * db + 4 * (p & 3));
+    const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(va));
+    const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) i16x4*)(va + 16 * G::kPitchV));
+    const u32x2 lo2 = __builtin_bit_cast(u32x2, lo), hi2 = __builtin_bit_cast(u32x2, hi);
+    const u32x4 vf = {lo2[0], lo2[1], hi2[0], hi2[1]};
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) st.o[qb][db] = E::mfma(vf, pf[qb], st.o[qb][db]);
+  }
+}
+
+// One wave attends NQB*16 query rows to tokens [tile0*32, ...) in steps of tile_step_n tiles,
+// staging each tile in its own LDS area.
+template <typename E, int D, int NQB, bool GATHERED>
+__device__ __forceinline__ void wave_attend(const Stage1Args& a, const VnodeView& vn, int kvh, int row0,
+                                            int tile0, int tile_step_n, char* lds, WaveState<D, NQB>& st) {
+  using G = TileGeom<D>;
+  const int lane = threadIdx.x & 63;
+  char* ldsK = lds;
+  char* ldsV = lds + G::kBytesK;
+
+  u32x4 qf[NQB][D / 32];
+  load_q_frags<D, NQB, GATHERED>(a, vn, kvh, row0, qf);
+  reset_state<D, NQB>(st);
 
   const int ntiles = (vn.kv_len + kTileTokens - 1) / kTileTokens;
   if (tile0 >= ntiles) return;
@@ -229,7 +341,7 @@ __device__ __forceinline__ void wave_attend(const Stage1Args& a, const VnodeView
   };
   fetch(tile0);
 
-  for (int tile = tile0; tile < ntiles; tile += tile_step) {
+  for (int tile = tile0; tile < ntiles; tile += tile_step_n) {
     // registers -> this wave's LDS tile
 #pragma unroll
     for (int i = 0; i < G::kLoads; ++i) {
@@ -238,76 +350,11 @@ __device__ __forceinline__ void wave_attend(const Stage1Args& a, const VnodeView
       *reinterpret_cast<u32x4*>(ldsV + row * G::kPitchV + 16 * ld_chunk) = vreg[i];
     }
     wave_lds_fence();
-    if (tile + tile_step < ntiles) fetch(tile + tile_step);
-
-    // ---- S^T = K Q^T : s[tb][qb][j] = score(token 16*tb + 4*c + j, row 16*qb + p)
-    f32x4 s[2][NQB];
-#pragma unroll
-    for (int tb = 0; tb < 2; ++tb) {
-#pragma unroll
-      for (int qb = 0; qb < NQB; ++qb) s[tb][qb] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const u32x4 kf = *reinterpret_cast<const u32x4*>(ldsK + (16 * tb + p) * G::kPitchK + 64 * ks + 16 * c);
-#pragma unroll
-        for (int qb = 0; qb < NQB; ++qb) s[tb][qb] = E::mfma(kf, qf[qb][ks], s[tb][qb]);
-      }
-    }
-
-    const int valid = vn.kv_len - tile * kTileTokens;  // tokens of this tile that exist
-    const float sc = a.scale_log2;
-    u32x4 pf[NQB];
-#pragma unroll
-    for (int qb = 0; qb < NQB; ++qb) {
-      float x[8];
-#pragma unroll
-      for (int tb = 0; tb < 2; ++tb)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          float val = s[tb][qb][j] * sc;
-          if (valid < kTileTokens && 16 * tb + 4 * c + j >= valid) val = -INFINITY;
-          x[4 * tb + j] = val;
-        }
-      float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
-      mx = xor32_max(xor16_max(mx));
-      const float m_old = st.m[qb];
-      const float m_new = fmaxf(m_old, mx);  // finite: every tile holds at least one token
-      float sum = 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        x[i] = __builtin_amdgcn_exp2f(x[i] - m_new);
-        sum += x[i];
-      }
-      if (__builtin_amdgcn_ballot_w64(m_new > m_old)) {  // wave-uniform: rescale only when a max moved
-        const float alpha = __builtin_amdgcn_exp2f(m_old - m_new);
-        st.l[qb] *= alpha;
-#pragma unroll
-        for (int db = 0; db < DB; ++db) st.o[qb][db] *= alpha;
-      }
-      st.l[qb] += sum;
-      st.m[qb] = m_new;
-      pf[qb] = u32x4{E::pack2(x[0], x[1]), E::pack2(x[2], x[3]), E::pack2(x[4], x[5]), E::pack2(x[6], x[7])};
-    }
-
-    // ---- O^T += V^T P^T : A operand rows = dims 16*db + p, k slots = the 8 tokens this lane's P holds
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      const char* va = ldsV + (4 * c + (p >> 2)) * G::kPitchV + 2 * (16 * db + 4 * (p & 3));
-      const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (__attribute__((address_space(3))) i16x4*)(va));
-      const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (__attribute__((address_space(3))) i16x4*)(va + 16 * G::kPitchV));
-      const u32x2 lo2 = __builtin_bit_cast(u32x2, lo), hi2 = __builtin_bit_cast(u32x2, hi);
-      const u32x4 vf = {lo2[0], lo2[1], hi2[0], hi2[1]};
-#pragma unroll
-      for (int qb = 0; qb < NQB; ++qb) st.o[qb][db] = E::mfma(vf, pf[qb], st.o[qb][db]);
-    }
+    if (tile + tile_step_n < ntiles) fetch(tile + tile_step_n);
+    tile_step<E, D, NQB>(ldsK, ldsV, vn.kv_len - tile * kTileTokens, a.scale_log2, qf, st);
     wave_lds_fence();
   }
-
-  // every lane of a row now gets the row's full probability sum
-#pragma unroll
-  for (int qb = 0; qb < NQB; ++qb) st.l[qb] = xor32_sum(xor16_sum(st.l[qb]));
+  finish_state<D, NQB>(st);
 }
 
 template <int D, int NQB>
@@ -330,6 +377,49 @@ __device__ __forceinline__ void write_partials(const Stage1Args& a, const VnodeV
 #pragma unroll
     for (int db = 0; db < DB; ++db) *reinterpret_cast<f32x4*>(dst + 16 * db) = st.o[qb][db] * inv;
     if (c == 0) a.mid_lse[row * a.sl0 + head] = l > 0.f ? (__builtin_amdgcn_logf(l) + st.m[qb]) * kLn2 : -INFINITY;
+  }
+}
+
+// Merge of the four waves' states of one block (each over the same rows, different tokens)
+// into wave 0, pairwise through LDS: waves {2,3} -> {0,1}, then wave 1 -> wave 0.
+template <int D, int NQB>
+__device__ __forceinline__ void merge_waves(float* xchg, WaveState<D, NQB>& st) {
+  constexpr int NV = NQB * (D / 16) * 4 + 2 * NQB;  // floats of state per lane
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll
+  for (int half = 2; half >= 1; half >>= 1) {
+    __syncthreads();
+    if (wave >= half && wave < 2 * half) {
+      float* dst = xchg + (size_t)(wave - half) * NV * kWave + lane;
+      int n = 0;
+#pragma unroll
+      for (int qb = 0; qb < NQB; ++qb) {
+        dst[(n++) * kWave] = st.m[qb];
+        dst[(n++) * kWave] = st.l[qb];
+#pragma unroll
+        for (int db = 0; db < D / 16; ++db)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) dst[(n++) * kWave] = st.o[qb][db][j];
+      }
+    }
+    __syncthreads();
+    if (wave < half) {
+      const float* src = xchg + (size_t)wave * NV * kWave + lane;
+      int n = 0;
+#pragma unroll
+      for (int qb = 0; qb < NQB; ++qb) {
+        const float m2 = src[(n++) * kWave];
+        const float l2 = src[(n++) * kWave];
+        const float m = fmaxf(st.m[qb], m2);
+        const float a1 = scale_from(st.m[qb], m), a2 = scale_from(m2, m);
+        st.l[qb] = st.l[qb] * a1 + l2 * a2;
+        st.m[qb] = m;
+#pragma unroll
+        for (int db = 0; db < D / 16; ++db)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) st.o[qb][db][j] = st.o[qb][db][j] * a1 + src[(n++) * kWave] * a2;
+      }
+    }
   }
 }
 
@@ -357,50 +447,349 @@ __global__ void __launch_bounds__(kBlock) stage1_kernel(Stage1Args a) {
   } else {
     const VnodeView vn = load_vnode<GATHERED>(a, a.vnode_begin + blockIdx.x);
     const int rows_total = vn.q_len * a.g;
-    constexpr int NV = NQB * (D / 16) * 4 + 2 * NQB;  // floats of state per lane
-    float* xchg = reinterpret_cast<float*>(smem);
     for (int row0 = 0; row0 < rows_total; row0 += 16 * NQB) {
       WaveState<D, NQB> st;
       wave_attend<E, D, NQB, GATHERED>(a, vn, kvh, row0, wave, kWavesPerBlock, my_lds, st);
-      // pairwise merge: waves {2,3} -> {0,1}, then wave 1 -> wave 0, through the staging LDS
-#pragma unroll
-      for (int half = 2; half >= 1; half >>= 1) {
-        __syncthreads();
-        if (wave >= half && wave < 2 * half) {
-          float* dst = xchg + (size_t)(wave - half) * NV * kWave + lane;
-          int n = 0;
-#pragma unroll
-          for (int qb = 0; qb < NQB; ++qb) {
-            dst[(n++) * kWave] = st.m[qb];
-            dst[(n++) * kWave] = st.l[qb];
-#pragma unroll
-            for (int db = 0; db < D / 16; ++db)
-#pragma unroll
-              for (int j = 0; j < 4; ++j) dst[(n++) * kWave] = st.o[qb][db][j];
-          }
-        }
-        __syncthreads();
-        if (wave < half) {
-          const float* src = xchg + (size_t)wave * NV * kWave + lane;
-          int n = 0;
-#pragma unroll
-          for (int qb = 0; qb < NQB; ++qb) {
-            const float m2 = src[(n++) * kWave];
-            const float l2 = src[(n++) * kWave];
-            const float m = fmaxf(st.m[qb], m2);
-            const float a1 = scale_from(st.m[qb], m), a2 = scale_from(m2, m);
-            st.l[qb] = st.l[qb] * a1 + l2 * a2;
-            st.m[qb] = m;
-#pragma unroll
-            for (int db = 0; db < D / 16; ++db)
-#pragma unroll
-              for (int j = 0; j < 4; ++j) st.o[qb][db][j] = st.o[qb][db][j] * a1 + src[(n++) * kWave] * a2;
-          }
-        }
-      }
+      merge_waves<D, NQB>(reinterpret_cast<float*>(smem), st);
       if (wave == 0) write_partials<D, NQB>(a, vn, kvh, row0, st);
       __syncthreads();  // staging LDS is reused by the next row chunk
     }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Wide vnodes: 32x32x16 MFMA tiles (twice the rate of 16x16x32 on this part).
+// ---------------------------------------------------------------------------------------
+
+// LDS layout of the wide kernel: rows of 2*D bytes back to back (no padding), 128-token super
+// tiles of four 32-token tiles, two buffers.  A row's 16-byte chunks are stored XOR-permuted:
+// chunk c of row r sits in slot c ^ swz(r).  swz swaps the two low bit pairs of r, which makes
+// both read patterns conflict free for 256-byte rows: the K operand read (16 different rows,
+// same chunk) and the transposed V read (4 consecutive rows x 4 consecutive chunks).
+// Loads go global -> LDS directly; one wave instruction fills a 1 KB group of consecutive rows.
+template <int D> struct WideGeom {
+  static constexpr int kRowBytes = 2 * D;
+  static constexpr int kChunks = D / 8;                  // 16-byte chunks per row
+  static constexpr int kSub = 4;
+  static constexpr int kTokens = kSub * kTileTokens;     // 128
+  static constexpr int kTileBytes = kTileTokens * kRowBytes;
+  static constexpr int kBytesK = kTokens * kRowBytes;
+  static constexpr int kBytes = 2 * kBytesK;             // K + V of one buffer
+  static constexpr int kGroupRows = kWave / kChunks;     // rows per 1 KB load group
+  static constexpr int kGroups = kTokens / kGroupRows;
+  static constexpr int kGroupsPerWave = kGroups / kWavesPerBlock;
+  static __device__ __forceinline__ int swz(int row) { return (((row & 3) << 2) | ((row >> 2) & 3)) & (kChunks - 1); }
+};
+
+// State of one wave for NQ blocks of 32 query rows.  o[qb][db][j] = O[row 32*qb + l%32]
+// [dim 32*db + 8*(j/4) + 4*(l/32) + j%4]; l is this lane's own share of the row sum.
+template <int D, int NQ> struct WideState {
+  f32x16 o[NQ][D / 32];
+  float m[NQ];
+  float l[NQ];
+};
+
+template <int D, int NQ>
+__device__ __forceinline__ void reset_state(WideState<D, NQ>& st) {
+#pragma unroll
+  for (int qb = 0; qb < NQ; ++qb) {
+    st.m[qb] = -INFINITY;
+    st.l[qb] = 0.f;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) st.o[qb][db][j] = 0.f;
+  }
+}
+
+// qf[qb][ks]: row row0 + 32*qb + lane%32, dims 16*ks + 8*(lane/32) .. +7; zero past the vnode.
+template <int D, int NQ, bool GATHERED>
+__device__ __forceinline__ void load_q_frags32(const Stage1Args& a, const VnodeView& vn, int kvh, int row0,
+                                               u32x4 (&qf)[NQ][D / 16]) {
+  const int lane = threadIdx.x & 63;
+  const int p = lane & 31, h = lane >> 5;
+  const int rows_total = vn.q_len * a.g;
+#pragma unroll
+  for (int qb = 0; qb < NQ; ++qb) {
+    const int r = row0 + 32 * qb + p;
+    const bool ok = r < rows_total;
+    const int ri = ok ? r / a.g : 0;
+    const int rj = ok ? r - ri * a.g : 0;
+    const int64_t entry = ok ? (GATHERED ? (int64_t)(vn.q_off / a.nsplit) : (int64_t)a.q_entries[vn.q_off + ri]) : 0;
+    const char* src = a.q + 2 * (entry * a.sq0 + (int64_t)(kvh * a.g + rj) * a.sq1 + 8 * h);
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      u32x4 z = {0u, 0u, 0u, 0u};
+      qf[qb][ks] = ok ? *reinterpret_cast<const u32x4*>(src + 32 * ks) : z;
+    }
+  }
+}
+
+// One 32-token step for 32*NQ rows.  S^T = K Q^T: A = K rows (token lane%32, 8 dims per lane),
+// B = Q; accumulator register j of a lane is token 8*(j/4) + 4*(lane/32) + j%4.  Registers
+// 8u .. 8u+7 are exactly the 8 k-slots a lane feeds to the u-th P.V contraction, whose A
+// operand (V^T) comes from two transposed LDS reads of 4 consecutive tokens each.
+template <typename E, int D, int NQ>
+__device__ __forceinline__ void tile_step32(const char* ldsK, const char* ldsV, int valid, float sc,
+                                            const u32x4 (&qf)[NQ][D / 16], WideState<D, NQ>& st) {
+  using W = WideGeom<D>;
+  constexpr int KS = D / 16, DB = D / 32;
+  const int lane = threadIdx.x & 63;
+  const int p32 = lane & 31, h = lane >> 5;
+
+  f32x16 s[NQ];
+#pragma unroll
+  for (int qb = 0; qb < NQ; ++qb)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) s[qb][j] = 0.f;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const u32x4 kf = *reinterpret_cast<const u32x4*>(ldsK + p32 * W::kRowBytes + 16 * ((2 * ks + h) ^ W::swz(p32)));
+#pragma unroll
+    for (int qb = 0; qb < NQ; ++qb) s[qb] = E::mfma32(kf, qf[qb][ks], s[qb]);
+  }
+
+  if (valid < kTileTokens) {  // wave-uniform: only the last tile of a run
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+      if (8 * (j >> 2) + 4 * h + (j & 3) >= valid) {
+#pragma unroll
+        for (int qb = 0; qb < NQ; ++qb) s[qb][j] = -INFINITY;
+      }
+  }
+
+  constexpr float kSlack = 8.f;  // lazily updated soft-max reference, see tile_step
+  u32x4 pf[NQ][2];
+#pragma unroll
+  for (int qb = 0; qb < NQ; ++qb) {
+    float mx = s[qb][0];
+#pragma unroll
+    for (int j = 1; j < 16; ++j) mx = fmaxf(mx, s[qb][j]);
+    mx = xor32_max(mx) * sc;
+    const float m_old = st.m[qb];
+    const bool grow = mx > m_old + kSlack;
+    if (__builtin_amdgcn_ballot_w64(grow)) {
+      const float m_new = grow ? mx : m_old;
+      const float alpha = __builtin_amdgcn_exp2f(m_old - m_new);
+      st.l[qb] *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) st.o[qb][db] *= alpha;
+      st.m[qb] = m_new;
+    }
+    const float neg_m = -st.m[qb];
+    float x[16];
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      x[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][j], sc, neg_m));
+      sum += x[j];
+    }
+    st.l[qb] += sum;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+      pf[qb][u] = u32x4{E::pack2(x[8 * u + 0], x[8 * u + 1]), E::pack2(x[8 * u + 2], x[8 * u + 3]),
+                        E::pack2(x[8 * u + 4], x[8 * u + 5]), E::pack2(x[8 * u + 6], x[8 * u + 7])};
+  }
+
+  const int p = lane & 15, gi = (lane >> 4) & 1;
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int row_lo = 16 * u + 4 * h + (p >> 2), row_hi = row_lo + 8;
+      const int chunk = 4 * db + 2 * gi + ((p & 3) >> 1);
+      const char* lo_at = ldsV + row_lo * W::kRowBytes + 16 * (chunk ^ W::swz(row_lo)) + 8 * (p & 1);
+      const char* hi_at = ldsV + row_hi * W::kRowBytes + 16 * (chunk ^ W::swz(row_hi)) + 8 * (p & 1);
+      const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(lo_at));
+      const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(hi_at));
+      const u32x2 lo2 = __builtin_bit_cast(u32x2, lo), hi2 = __builtin_bit_cast(u32x2, hi);
+      const u32x4 vf = {lo2[0], lo2[1], hi2[0], hi2[1]};
+#pragma unroll
+      for (int qb = 0; qb < NQ; ++qb) st.o[qb][db] = E::mfma32(vf, pf[qb][u], st.o[qb][db]);
+    }
+}
+
+template <int D, int NQ>
+__device__ __forceinline__ void finish_state(WideState<D, NQ>& st) {
+#pragma unroll
+  for (int qb = 0; qb < NQ; ++qb) st.l[qb] = xor32_sum(st.l[qb]);
+}
+
+template <int D, int NQ>
+__device__ __forceinline__ void write_partials32(const Stage1Args& a, const VnodeView& vn, int kvh, int row0,
+                                                 const WideState<D, NQ>& st) {
+  const int lane = threadIdx.x & 63;
+  const int p = lane & 31, h = lane >> 5;
+  const int rows_total = vn.q_len * a.g;
+#pragma unroll
+  for (int qb = 0; qb < NQ; ++qb) {
+    const int r = row0 + 32 * qb + p;
+    if (r >= rows_total) continue;
+    const int ri = r / a.g, rj = r - ri * a.g;
+    const int64_t row = vn.q_off + ri;
+    const int head = kvh * a.g + rj;
+    const float l = st.l[qb];
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    float* dst = a.mid_o + row * a.so0 + (int64_t)head * a.so1 + 4 * h;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const f32x4 v = {st.o[qb][db][4 * jj] * inv, st.o[qb][db][4 * jj + 1] * inv, st.o[qb][db][4 * jj + 2] * inv,
+                         st.o[qb][db][4 * jj + 3] * inv};
+        *reinterpret_cast<f32x4*>(dst + 32 * db + 8 * jj) = v;
+      }
+    if (h == 0) a.mid_lse[row * a.sl0 + head] = l > 0.f ? (__builtin_amdgcn_logf(l) + st.m[qb]) * kLn2 : -INFINITY;
+  }
+}
+
+// Merge of the four waves' states (same rows, different tokens) into wave 0 through LDS.
+template <int D, int NQ>
+__device__ __forceinline__ void merge_waves(float* xchg, WideState<D, NQ>& st) {
+  constexpr int NV = NQ * (D / 32) * 16 + 2 * NQ;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll
+  for (int half = 2; half >= 1; half >>= 1) {
+    __syncthreads();
+    if (wave >= half && wave < 2 * half) {
+      float* dst = xchg + (size_t)(wave - half) * NV * kWave + lane;
+      int n = 0;
+#pragma unroll
+      for (int qb = 0; qb < NQ; ++qb) {
+        dst[(n++) * kWave] = st.m[qb];
+        dst[(n++) * kWave] = st.l[qb];
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+          for (int j = 0; j < 16; ++j) dst[(n++) * kWave] = st.o[qb][db][j];
+      }
+    }
+    __syncthreads();
+    if (wave < half) {
+      const float* src = xchg + (size_t)wave * NV * kWave + lane;
+      int n = 0;
+#pragma unroll
+      for (int qb = 0; qb < NQ; ++qb) {
+        const float m2 = src[(n++) * kWave];
+        const float l2 = src[(n++) * kWave];
+        const float m = fmaxf(st.m[qb], m2);
+        const float a1 = scale_from(st.m[qb], m), a2 = scale_from(m2, m);
+        st.l[qb] = st.l[qb] * a1 + l2 * a2;
+        st.m[qb] = m;
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+          for (int j = 0; j < 16; ++j) st.o[qb][db][j] = st.o[qb][db][j] * a1 + src[(n++) * kWave] * a2;
+      }
+    }
+  }
+}
+
+// One block per (vnode, kv head).  The block streams the vnode's KV run through LDS 128 tokens
+// at a time with direct global->LDS loads (no staging registers); the next super tile is in
+// flight while the current one is consumed.  Up to 4*32*NQ query rows are served per pass over
+// the run: each wave owns 32*NQ of them and consumes every tile ("row split").  When no more
+// than 32*NQ rows are left the four waves instead share those rows and each consumes one of the
+// four tiles of a super tile ("token split"); their states are merged at the end.
+template <typename E, int D, int NQ, bool GATHERED>
+__global__ void __launch_bounds__(kBlock) stage1_dense_kernel(Stage1Args a) {
+  using W = WideGeom<D>;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int kvh = blockIdx.y;
+  const VnodeView vn = load_vnode<GATHERED>(a, a.vnode_begin + blockIdx.x);
+  const int rows_total = vn.q_len * a.g;
+  const int nsuper = (vn.kv_len + W::kTokens - 1) / W::kTokens;
+  constexpr int kWaveRows = 32 * NQ;
+
+  // loader role of this lane: 16-byte slot `pos` of row `grp_row` in each 1 KB group it fills
+  const int grp_row = lane / W::kChunks, pos = lane % W::kChunks;
+  const char* kbase = a.k + 2 * ((int64_t)kvh * a.sk1);
+  const char* vbase = a.v + 2 * ((int64_t)kvh * a.sv1);
+
+  for (int row0 = 0; row0 < rows_total;) {
+    const bool token_split = rows_total - row0 <= kWaveRows;
+    const int my_row0 = token_split ? row0 : row0 + wave * kWaveRows;
+    const bool has_rows = my_row0 < rows_total;
+
+    u32x4 qf[NQ][D / 16];
+    load_q_frags32<D, NQ, GATHERED>(a, vn, kvh, my_row0, qf);
+    WideState<D, NQ> st;
+    reset_state<D, NQ>(st);
+
+    // slots of the rows this lane loads in the next super tile (group g = j*4 + wave)
+    int slot[W::kGroupsPerWave];
+    auto load_slots = [&](int super) {
+#pragma unroll
+      for (int j = 0; j < W::kGroupsPerWave; ++j) {
+        const int t = super * W::kTokens + (j * kWavesPerBlock + wave) * W::kGroupRows + grp_row;
+        slot[j] = -1;
+        if (t < vn.kv_len) slot[j] = GATHERED ? (int)t : a.kv_entries[vn.kv_base + t];
+      }
+    };
+    auto issue_rows = [&](int super) {
+      char* bufK = smem + (super & 1) * W::kBytes;
+      char* bufV = bufK + W::kBytesK;
+#pragma unroll
+      for (int j = 0; j < W::kGroupsPerWave; ++j) {
+        const int grp = j * kWavesPerBlock + wave;
+        const int row = grp * W::kGroupRows + grp_row;
+        const int chunk = pos ^ W::swz(row);
+        char* dstK = bufK + grp * 1024;   // wave-uniform; lane l lands at +16*l
+        char* dstV = bufV + grp * 1024;
+        if (slot[j] >= 0) {
+          const int64_t srow = GATHERED ? (vn.kv_base + slot[j]) : (int64_t)slot[j];
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kbase + 2 * srow * a.sk0 + 16 * chunk),
+                                           (__attribute__((address_space(3))) void*)dstK, 16, 0, 0);
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vbase + 2 * srow * a.sv0 + 16 * chunk),
+                                           (__attribute__((address_space(3))) void*)dstV, 16, 0, 0);
+        } else {
+          // rows past the run: V must be finite (it meets zero probabilities), K is masked later
+          *reinterpret_cast<u32x4*>(dstV + 16 * lane) = u32x4{0u, 0u, 0u, 0u};
+        }
+      }
+    };
+    if (nsuper > 0) {
+      load_slots(0);
+      issue_rows(0);
+      if (nsuper > 1) load_slots(1);
+    }
+    for (int super = 0; super < nsuper; ++super) {
+      // the loads of this super tile were issued one iteration ago; publish them to the block
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      __syncthreads();
+      // the other buffer was last read before that barrier: refill it now
+      if (super + 1 < nsuper) {
+        issue_rows(super + 1);
+        if (super + 2 < nsuper) load_slots(super + 2);
+      }
+      const char* bufK = smem + (super & 1) * W::kBytes;
+      const char* bufV = bufK + W::kBytesK;
+      if (has_rows) {
+        const int left = vn.kv_len - super * W::kTokens;  // tokens from the start of this super tile
+        if (token_split) {
+          const int valid = left - wave * kTileTokens;
+          if (valid > 0)
+            tile_step32<E, D, NQ>(bufK + wave * W::kTileBytes, bufV + wave * W::kTileBytes, valid, a.scale_log2, qf, st);
+        } else {
+#pragma unroll 1
+          for (int sub = 0; sub < W::kSub; ++sub) {
+            const int valid = left - sub * kTileTokens;
+            if (valid > 0)
+              tile_step32<E, D, NQ>(bufK + sub * W::kTileBytes, bufV + sub * W::kTileBytes, valid, a.scale_log2, qf, st);
+          }
+        }
+      }
+    }
+    finish_state<D, NQ>(st);
+    if (token_split) {
+      merge_waves<D, NQ>(reinterpret_cast<float*>(smem), st);
+      if (wave == 0) write_partials32<D, NQ>(a, vn, kvh, my_row0, st);
+    } else if (has_rows) {
+      write_partials32<D, NQ>(a, vn, kvh, my_row0, st);
+    }
+    __syncthreads();  // staging LDS is reused by the next pass over the run
+    row0 += token_split ? kWaveRows : kWavesPerBlock * kWaveRows;
   }
 }
 
@@ -501,13 +890,34 @@ int launch_stage1_inst(const Stage1Args& a, int hkv, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? FT_OK : FT_ERR_LAUNCH;
 }
 
+template <typename E, int D, int NQ, bool GATHERED>
+int launch_stage1_dense(const Stage1Args& a, int hkv, hipStream_t stream) {
+  const size_t lds = 2 * (size_t)WideGeom<D>::kBytes;
+  auto kern = stage1_dense_kernel<E, D, NQ, GATHERED>;
+  static bool configured = false;
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+      (void)hipGetLastError();
+      return FT_ERR_LAUNCH;
+    }
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)a.vnode_count, (unsigned)hkv, 1), dim3(kBlock, 1, 1), lds, stream, a);
+  return hipGetLastError() == hipSuccess ? FT_OK : FT_ERR_LAUNCH;
+}
+
 template <typename E, int D, bool GATHERED>
 int launch_stage1_d(const Stage1Args& a, int hkv, int rows_per_vnode, hipStream_t stream) {
-  // Row blocks per wave: enough for the phase's tile, at most 64 rows (wider vnodes loop).
-  constexpr int kMaxNqb = D > 128 ? 2 : 4;
+  // Narrow vnodes (<= 16 rows): one wave each.  Wider: one block each, 32 or 64 rows per wave
+  // and up to four waves' worth of rows per pass over the KV run.
   if (rows_per_vnode <= 16) return launch_stage1_inst<E, D, 1, false, GATHERED>(a, hkv, stream);
-  if (rows_per_vnode <= 32 || kMaxNqb == 2) return launch_stage1_inst<E, D, 2, true, GATHERED>(a, hkv, stream);
-  return launch_stage1_inst<E, D, kMaxNqb, true, GATHERED>(a, hkv, stream);
+  if constexpr (D > 128) {
+    // 128-token double buffers of 256-wide rows do not fit in LDS: per-wave staging instead
+    return launch_stage1_inst<E, D, 2, true, GATHERED>(a, hkv, stream);
+  } else {
+    if (rows_per_vnode <= 32) return launch_stage1_dense<E, D, 1, GATHERED>(a, hkv, stream);
+    return launch_stage1_dense<E, D, 2, GATHERED>(a, hkv, stream);
+  }
 }
 
 template <bool GATHERED>
