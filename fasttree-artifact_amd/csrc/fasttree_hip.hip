@@ -91,6 +91,7 @@ __device__ __forceinline__ float xor16_max(float x) { LanePair h = halves16(x); 
 __device__ __forceinline__ float xor32_max(float x) { LanePair h = halves32(x); return fmaxf(h.lo, h.hi); }
 __device__ __forceinline__ float xor16_sum(float x) { LanePair h = halves16(x); return h.lo + h.hi; }
 __device__ __forceinline__ float xor32_sum(float x) { LanePair h = halves32(x); return h.lo + h.hi; }
+__device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
 // Orders this wave's LDS traffic around a point where lanes read what other lanes of the
 // same wave wrote.  LDS executes one wave's instructions in order, so no wait is needed;
 // the fences only stop the compiler from moving accesses across.
@@ -458,8 +459,21 @@ __global__ void __launch_bounds__(kBlock) stage1_kernel(Stage1Args a) {
 }
 
 // ---------------------------------------------------------------------------------------
-// Wide vnodes: 32x32x16 MFMA tiles (twice the rate of 16x16x32 on this part).
+// Wide vnodes: 32x32x16 MFMA tiles (twice the rate of 16x16x32 on this part), 8 waves per
+// block with 32 query rows each, so that two waves share a SIMD and one wave's soft-max
+// arithmetic overlaps the other's matrix instructions.
 // ---------------------------------------------------------------------------------------
+#ifdef FT_TIMING
+// Development aid, compiled out of the product: per-wave cycle counts of the wide kernel's
+// phases, written to a buffer set with ft_debug_set_timing().
+__device__ unsigned long long* g_timing = nullptr;
+#define FT_CLOCK() __builtin_readcyclecounter()
+#define FT_TIME(...) __VA_ARGS__
+#else
+#define FT_TIME(...)
+#endif
+constexpr int kWideWaves = 8;
+constexpr int kWideBlock = kWave * kWideWaves;
 
 // LDS layout of the wide kernel: rows of 2*D bytes back to back (no padding), 128-token super
 // tiles of four 32-token tiles, two buffers.  A row's 16-byte chunks are stored XOR-permuted:
@@ -474,225 +488,235 @@ template <int D> struct WideGeom {
   static constexpr int kTokens = kSub * kTileTokens;     // 128
   static constexpr int kTileBytes = kTileTokens * kRowBytes;
   static constexpr int kBytesK = kTokens * kRowBytes;
-  static constexpr int kBytes = 2 * kBytesK;             // K + V of one buffer
+  static constexpr int kBytes = 2 * kBytesK;             // K + V of one buffer (a power of two)
   static constexpr int kGroupRows = kWave / kChunks;     // rows per 1 KB load group
   static constexpr int kGroups = kTokens / kGroupRows;
-  static constexpr int kGroupsPerWave = kGroups / kWavesPerBlock;
+  static constexpr int kGroupsPerWave = kGroups / kWideWaves;
   static __device__ __forceinline__ int swz(int row) { return (((row & 3) << 2) | ((row >> 2) & 3)) & (kChunks - 1); }
 };
 
-// State of one wave for NQ blocks of 32 query rows.  o[qb][db][j] = O[row 32*qb + l%32]
-// [dim 32*db + 8*(j/4) + 4*(l/32) + j%4]; l is this lane's own share of the row sum.
-template <int D, int NQ> struct WideState {
-  f32x16 o[NQ][D / 32];
-  float m[NQ];
-  float l[NQ];
+// State of one wave for its 32 query rows.  o[db][j] = O[row lane%32][dim 32*db + 8*(j/4) +
+// 4*(lane/32) + j%4]; m = soft-max reference (scaled scores, log2 domain); l = this lane's own
+// share of the row sum until finish_state().
+template <int D> struct WideState {
+  f32x16 o[D / 32];
+  float m;
+  float l;
 };
 
-template <int D, int NQ>
-__device__ __forceinline__ void reset_state(WideState<D, NQ>& st) {
+template <int D>
+__device__ __forceinline__ void reset_state(WideState<D>& st) {
+  st.m = -INFINITY;
+  st.l = 0.f;
 #pragma unroll
-  for (int qb = 0; qb < NQ; ++qb) {
-    st.m[qb] = -INFINITY;
-    st.l[qb] = 0.f;
+  for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-    for (int db = 0; db < D / 32; ++db)
-#pragma unroll
-      for (int j = 0; j < 16; ++j) st.o[qb][db][j] = 0.f;
-  }
+    for (int j = 0; j < 16; ++j) st.o[db][j] = 0.f;
 }
 
-// qf[qb][ks]: row row0 + 32*qb + lane%32, dims 16*ks + 8*(lane/32) .. +7; zero past the vnode.
-template <int D, int NQ, bool GATHERED>
+// qf[ks]: row row0 + lane%32, dims 16*ks + 8*(lane/32) .. +7; zero past the vnode.
+template <int D, bool GATHERED>
 __device__ __forceinline__ void load_q_frags32(const Stage1Args& a, const VnodeView& vn, int kvh, int row0,
-                                               u32x4 (&qf)[NQ][D / 16]) {
+                                               u32x4 (&qf)[D / 16]) {
   const int lane = threadIdx.x & 63;
-  const int p = lane & 31, h = lane >> 5;
-  const int rows_total = vn.q_len * a.g;
+  const int r = row0 + (lane & 31), h = lane >> 5;
+  const bool ok = r < vn.q_len * a.g;
+  const int ri = ok ? r / a.g : 0;
+  const int rj = ok ? r - ri * a.g : 0;
+  const int64_t entry = ok ? (GATHERED ? (int64_t)(vn.q_off / a.nsplit) : (int64_t)a.q_entries[vn.q_off + ri]) : 0;
+  const char* src = a.q + 2 * (entry * a.sq0 + (int64_t)(kvh * a.g + rj) * a.sq1 + 8 * h);
 #pragma unroll
-  for (int qb = 0; qb < NQ; ++qb) {
-    const int r = row0 + 32 * qb + p;
-    const bool ok = r < rows_total;
-    const int ri = ok ? r / a.g : 0;
-    const int rj = ok ? r - ri * a.g : 0;
-    const int64_t entry = ok ? (GATHERED ? (int64_t)(vn.q_off / a.nsplit) : (int64_t)a.q_entries[vn.q_off + ri]) : 0;
-    const char* src = a.q + 2 * (entry * a.sq0 + (int64_t)(kvh * a.g + rj) * a.sq1 + 8 * h);
-#pragma unroll
-    for (int ks = 0; ks < D / 16; ++ks) {
-      u32x4 z = {0u, 0u, 0u, 0u};
-      qf[qb][ks] = ok ? *reinterpret_cast<const u32x4*>(src + 32 * ks) : z;
-    }
+  for (int ks = 0; ks < D / 16; ++ks) {
+    u32x4 z = {0u, 0u, 0u, 0u};
+    qf[ks] = ok ? *reinterpret_cast<const u32x4*>(src + 32 * ks) : z;
   }
 }
 
-// One 32-token step for 32*NQ rows.  S^T = K Q^T: A = K rows (token lane%32, 8 dims per lane),
-// B = Q; accumulator register j of a lane is token 8*(j/4) + 4*(lane/32) + j%4.  Registers
-// 8u .. 8u+7 are exactly the 8 k-slots a lane feeds to the u-th P.V contraction, whose A
-// operand (V^T) comes from two transposed LDS reads of 4 consecutive tokens each.
-template <typename E, int D, int NQ>
-__device__ __forceinline__ void tile_step32(const char* ldsK, const char* ldsV, int valid, float sc,
-                                            const u32x4 (&qf)[NQ][D / 16], WideState<D, NQ>& st) {
+// Per-lane LDS byte addresses of the operand reads inside tile 0 of buffer 0, for contraction
+// step / dim block 0.  Thanks to the XOR layout the address for step ks (dim block db) is the
+// base with 32*ks (64*db) XOR-ed in; other tiles of the super tile are a constant offset away
+// and the other buffer is reached by flipping bit log2(kBytes) (the buffers are kBytes apart,
+// kBytes is a power of two and the dynamic LDS segment starts at 0).
+struct WideLane {
+  unsigned k;     // K operand: row lane%32, chunk lane/32 (step ks: chunk 2*ks + lane/32)
+  unsigned v_lo;  // transposed V read: tokens 4*(lane/32) + 0..3 (+16 for u = 1), dims 0..31
+  unsigned v_hi;  // same, tokens + 8
+};
+
+template <int D>
+__device__ __forceinline__ void init_lane(WideLane& la) {
   using W = WideGeom<D>;
-  constexpr int KS = D / 16, DB = D / 32;
   const int lane = threadIdx.x & 63;
-  const int p32 = lane & 31, h = lane >> 5;
+  const int p32 = lane & 31, h = lane >> 5, p = lane & 15, gi = (lane >> 4) & 1;
+  la.k = p32 * W::kRowBytes + 16 * ((h & (W::kChunks - 1)) ^ W::swz(p32));
+  const int row_lo = 4 * h + (p >> 2), row_hi = row_lo + 8;
+  const int chunk = (2 * gi + ((p & 3) >> 1)) & (W::kChunks - 1);
+  la.v_lo = W::kBytesK + row_lo * W::kRowBytes + 16 * (chunk ^ W::swz(row_lo)) + 8 * (p & 1);
+  la.v_hi = W::kBytesK + row_hi * W::kRowBytes + 16 * (chunk ^ W::swz(row_hi)) + 8 * (p & 1);
+}
 
-  f32x16 s[NQ];
+template <int D>
+__device__ __forceinline__ void flip_buffer(WideLane& la) {
+  using W = WideGeom<D>;
+  la.k ^= W::kBytes;
+  la.v_lo ^= W::kBytes;
+  la.v_hi ^= W::kBytes;
+}
+
+__device__ __forceinline__ u32x4 lds_read16(unsigned addr) {
+  return *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>((uintptr_t)addr);
+}
+__device__ __forceinline__ u32x2 lds_read_tr8(unsigned addr) {
+  const i16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      reinterpret_cast<__attribute__((address_space(3))) i16x4*>((uintptr_t)addr));
+  return __builtin_bit_cast(u32x2, v);
+}
+
+// The soft-max reference m of a row is updated lazily: only when the row's running maximum
+// exceeds it by more than kSlack (log2 units).  Probabilities therefore stay below 2^kSlack --
+// exact in any case, since numerator and denominator share the reference -- and the
+// accumulators are rescaled rarely (in practice once, on a run's first tile).
+constexpr float kSlack = 8.f;
+
+// One 32-token step for the wave's 32 rows on the tile `off` bytes into the current buffer.
+// S^T = K Q^T: A = K rows (token lane%32, 8 dims per lane), B = Q; accumulator register j of a
+// lane is token 8*(j/4) + 4*(lane/32) + j%4.  Registers 8u .. 8u+7 are exactly the 8 k-slots a
+// lane feeds to the u-th P.V contraction, whose A operand (V^T) comes from two transposed LDS
+// reads of 4 consecutive tokens each.  MASKED is used for a run's last, partial tile only.
+template <typename E, int D, bool MASKED>
+__device__ __forceinline__ void tile_step32(const WideLane& la, unsigned off, int valid, float sc,
+                                            const u32x4 (&qf)[D / 16], WideState<D>& st) {
+  using W = WideGeom<D>;
+  constexpr int KS = D / 16, DB = D / 32, NV = 2 * DB;
+
+  // all K operands of the tile are requested before the first contraction needs one
+  const unsigned kb = la.k + off;
+  u32x4 kf[KS];
 #pragma unroll
-  for (int qb = 0; qb < NQ; ++qb)
+  for (int ks = 0; ks < KS; ++ks) kf[ks] = lds_read16(kb ^ (32u * ks));
+  f32x16 s;
 #pragma unroll
-    for (int j = 0; j < 16; ++j) s[qb][j] = 0.f;
+  for (int j = 0; j < 16; ++j) s[j] = 0.f;
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    const u32x4 kf = *reinterpret_cast<const u32x4*>(ldsK + p32 * W::kRowBytes + 16 * ((2 * ks + h) ^ W::swz(p32)));
+  for (int ks = 0; ks < KS; ++ks) s = E::mfma32(kf[ks], qf[ks], s);
+
+  if constexpr (MASKED) {
+    const int h = (threadIdx.x & 63) >> 5;
 #pragma unroll
-    for (int qb = 0; qb < NQ; ++qb) s[qb] = E::mfma32(kf, qf[qb][ks], s[qb]);
+    for (int j = 0; j < 16; ++j) s[j] = (8 * (j >> 2) + 4 * h + (j & 3) >= valid) ? -INFINITY : s[j];
   }
 
-  if (valid < kTileTokens) {  // wave-uniform: only the last tile of a run
+  float mx = max3(s[0], s[1], s[2]);
 #pragma unroll
-    for (int j = 0; j < 16; ++j)
-      if (8 * (j >> 2) + 4 * h + (j & 3) >= valid) {
+  for (int j = 3; j < 15; j += 2) mx = max3(mx, s[j], s[j + 1]);
+  mx = xor32_max(fmaxf(mx, s[15])) * sc;  // sc > 0; finite: the tile holds at least one token
+  const bool grow = mx > st.m + kSlack;   // also true on a run's first tile (m = -inf)
+  if (__builtin_amdgcn_ballot_w64(grow)) {
+    const float m_new = grow ? mx : st.m;
+    const float alpha = __builtin_amdgcn_exp2f(st.m - m_new);
+    st.l *= alpha;
 #pragma unroll
-        for (int qb = 0; qb < NQ; ++qb) s[qb][j] = -INFINITY;
-      }
+    for (int db = 0; db < DB; ++db) st.o[db] *= alpha;
+    st.m = m_new;
   }
 
-  constexpr float kSlack = 8.f;  // lazily updated soft-max reference, see tile_step
-  u32x4 pf[NQ][2];
+  const float neg_m = -st.m;
+  float x[16];
+  float sum = 0.f;
 #pragma unroll
-  for (int qb = 0; qb < NQ; ++qb) {
-    float mx = s[qb][0];
-#pragma unroll
-    for (int j = 1; j < 16; ++j) mx = fmaxf(mx, s[qb][j]);
-    mx = xor32_max(mx) * sc;
-    const float m_old = st.m[qb];
-    const bool grow = mx > m_old + kSlack;
-    if (__builtin_amdgcn_ballot_w64(grow)) {
-      const float m_new = grow ? mx : m_old;
-      const float alpha = __builtin_amdgcn_exp2f(m_old - m_new);
-      st.l[qb] *= alpha;
-#pragma unroll
-      for (int db = 0; db < DB; ++db) st.o[qb][db] *= alpha;
-      st.m[qb] = m_new;
-    }
-    const float neg_m = -st.m[qb];
-    float x[16];
-    float sum = 0.f;
-#pragma unroll
-    for (int j = 0; j < 16; ++j) {
-      x[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][j], sc, neg_m));
-      sum += x[j];
-    }
-    st.l[qb] += sum;
-#pragma unroll
-    for (int u = 0; u < 2; ++u)
-      pf[qb][u] = u32x4{E::pack2(x[8 * u + 0], x[8 * u + 1]), E::pack2(x[8 * u + 2], x[8 * u + 3]),
-                        E::pack2(x[8 * u + 4], x[8 * u + 5]), E::pack2(x[8 * u + 6], x[8 * u + 7])};
+  for (int j = 0; j < 16; ++j) {
+    x[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j], sc, neg_m));
+    sum += x[j];
   }
-
-  const int p = lane & 15, gi = (lane >> 4) & 1;
+  st.l += sum;
+  u32x4 pf[2];
 #pragma unroll
   for (int u = 0; u < 2; ++u)
+    pf[u] = u32x4{E::pack2(x[8 * u + 0], x[8 * u + 1]), E::pack2(x[8 * u + 2], x[8 * u + 3]),
+                  E::pack2(x[8 * u + 4], x[8 * u + 5]), E::pack2(x[8 * u + 6], x[8 * u + 7])};
+
+  const unsigned vlo = la.v_lo + off, vhi = la.v_hi + off;
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      const int row_lo = 16 * u + 4 * h + (p >> 2), row_hi = row_lo + 8;
-      const int chunk = 4 * db + 2 * gi + ((p & 3) >> 1);
-      const char* lo_at = ldsV + row_lo * W::kRowBytes + 16 * (chunk ^ W::swz(row_lo)) + 8 * (p & 1);
-      const char* hi_at = ldsV + row_hi * W::kRowBytes + 16 * (chunk ^ W::swz(row_hi)) + 8 * (p & 1);
-      const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(lo_at));
-      const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(hi_at));
-      const u32x2 lo2 = __builtin_bit_cast(u32x2, lo), hi2 = __builtin_bit_cast(u32x2, hi);
-      const u32x4 vf = {lo2[0], lo2[1], hi2[0], hi2[1]};
-#pragma unroll
-      for (int qb = 0; qb < NQ; ++qb) st.o[qb][db] = E::mfma32(vf, pf[qb][u], st.o[qb][db]);
-    }
+  for (int i = 0; i < NV; ++i) {
+    const int u = i / DB, db = i % DB;
+    const u32x2 lo = lds_read_tr8((vlo ^ (64u * db)) + u * 16 * W::kRowBytes);
+    const u32x2 hi = lds_read_tr8((vhi ^ (64u * db)) + u * 16 * W::kRowBytes);
+    const u32x4 vf = {lo[0], lo[1], hi[0], hi[1]};
+    st.o[db] = E::mfma32(vf, pf[u], st.o[db]);
+  }
 }
 
-template <int D, int NQ>
-__device__ __forceinline__ void finish_state(WideState<D, NQ>& st) {
-#pragma unroll
-  for (int qb = 0; qb < NQ; ++qb) st.l[qb] = xor32_sum(st.l[qb]);
+template <int D>
+__device__ __forceinline__ void finish_state(WideState<D>& st) {
+  st.l = xor32_sum(st.l);
 }
 
-template <int D, int NQ>
+template <int D>
 __device__ __forceinline__ void write_partials32(const Stage1Args& a, const VnodeView& vn, int kvh, int row0,
-                                                 const WideState<D, NQ>& st) {
+                                                 const WideState<D>& st) {
   const int lane = threadIdx.x & 63;
-  const int p = lane & 31, h = lane >> 5;
-  const int rows_total = vn.q_len * a.g;
+  const int r = row0 + (lane & 31), h = lane >> 5;
+  if (r >= vn.q_len * a.g) return;
+  const int ri = r / a.g, rj = r - ri * a.g;
+  const int64_t row = vn.q_off + ri;
+  const int head = kvh * a.g + rj;
+  const float inv = st.l > 0.f ? 1.f / st.l : 0.f;
+  float* dst = a.mid_o + row * a.so0 + (int64_t)head * a.so1 + 4 * h;
 #pragma unroll
-  for (int qb = 0; qb < NQ; ++qb) {
-    const int r = row0 + 32 * qb + p;
-    if (r >= rows_total) continue;
-    const int ri = r / a.g, rj = r - ri * a.g;
-    const int64_t row = vn.q_off + ri;
-    const int head = kvh * a.g + rj;
-    const float l = st.l[qb];
-    const float inv = l > 0.f ? 1.f / l : 0.f;
-    float* dst = a.mid_o + row * a.so0 + (int64_t)head * a.so1 + 4 * h;
+  for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-    for (int db = 0; db < D / 32; ++db)
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        const f32x4 v = {st.o[qb][db][4 * jj] * inv, st.o[qb][db][4 * jj + 1] * inv, st.o[qb][db][4 * jj + 2] * inv,
-                         st.o[qb][db][4 * jj + 3] * inv};
-        *reinterpret_cast<f32x4*>(dst + 32 * db + 8 * jj) = v;
-      }
-    if (h == 0) a.mid_lse[row * a.sl0 + head] = l > 0.f ? (__builtin_amdgcn_logf(l) + st.m[qb]) * kLn2 : -INFINITY;
-  }
+    for (int jj = 0; jj < 4; ++jj) {
+      const f32x4 v = {st.o[db][4 * jj] * inv, st.o[db][4 * jj + 1] * inv, st.o[db][4 * jj + 2] * inv,
+                       st.o[db][4 * jj + 3] * inv};
+      *reinterpret_cast<f32x4*>(dst + 32 * db + 8 * jj) = v;
+    }
+  if (h == 0) a.mid_lse[row * a.sl0 + head] = st.l > 0.f ? (__builtin_amdgcn_logf(st.l) + st.m) * kLn2 : -INFINITY;
 }
 
-// Merge of the four waves' states (same rows, different tokens) into wave 0 through LDS.
-template <int D, int NQ>
-__device__ __forceinline__ void merge_waves(float* xchg, WideState<D, NQ>& st) {
-  constexpr int NV = NQ * (D / 32) * 16 + 2 * NQ;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-#pragma unroll
-  for (int half = 2; half >= 1; half >>= 1) {
+// Merge of the TG waves that hold the same rows (token groups 0..TG-1 of row group rg) into
+// token group 0, pairwise through LDS.  Every wave of the block must call this.
+template <int D>
+__device__ __forceinline__ void merge_token_groups(float* xchg, WideState<D>& st, int rg, int tg, int tgroups, bool active) {
+  constexpr int NV = (D / 32) * 16 + 2;
+  const int lane = threadIdx.x & 63;
+  for (int half = tgroups >> 1; half >= 1; half >>= 1) {
     __syncthreads();
-    if (wave >= half && wave < 2 * half) {
-      float* dst = xchg + (size_t)(wave - half) * NV * kWave + lane;
+    if (active && tg >= half && tg < 2 * half) {
+      float* dst = xchg + (size_t)(rg * half + tg - half) * NV * kWave + lane;
       int n = 0;
+      dst[(n++) * kWave] = st.m;
+      dst[(n++) * kWave] = st.l;
 #pragma unroll
-      for (int qb = 0; qb < NQ; ++qb) {
-        dst[(n++) * kWave] = st.m[qb];
-        dst[(n++) * kWave] = st.l[qb];
+      for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-        for (int db = 0; db < D / 32; ++db)
-#pragma unroll
-          for (int j = 0; j < 16; ++j) dst[(n++) * kWave] = st.o[qb][db][j];
-      }
+        for (int j = 0; j < 16; ++j) dst[(n++) * kWave] = st.o[db][j];
     }
     __syncthreads();
-    if (wave < half) {
-      const float* src = xchg + (size_t)wave * NV * kWave + lane;
+    if (active && tg < half) {
+      const float* src = xchg + (size_t)(rg * half + tg) * NV * kWave + lane;
       int n = 0;
+      const float m2 = src[(n++) * kWave];
+      const float l2 = src[(n++) * kWave];
+      const float m = fmaxf(st.m, m2);
+      const float a1 = scale_from(st.m, m), a2 = scale_from(m2, m);
+      st.l = st.l * a1 + l2 * a2;
+      st.m = m;
 #pragma unroll
-      for (int qb = 0; qb < NQ; ++qb) {
-        const float m2 = src[(n++) * kWave];
-        const float l2 = src[(n++) * kWave];
-        const float m = fmaxf(st.m[qb], m2);
-        const float a1 = scale_from(st.m[qb], m), a2 = scale_from(m2, m);
-        st.l[qb] = st.l[qb] * a1 + l2 * a2;
-        st.m[qb] = m;
+      for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-        for (int db = 0; db < D / 32; ++db)
-#pragma unroll
-          for (int j = 0; j < 16; ++j) st.o[qb][db][j] = st.o[qb][db][j] * a1 + src[(n++) * kWave] * a2;
-      }
+        for (int j = 0; j < 16; ++j) st.o[db][j] = st.o[db][j] * a1 + src[(n++) * kWave] * a2;
     }
   }
 }
 
-// One block per (vnode, kv head).  The block streams the vnode's KV run through LDS 128 tokens
-// at a time with direct global->LDS loads (no staging registers); the next super tile is in
-// flight while the current one is consumed.  Up to 4*32*NQ query rows are served per pass over
-// the run: each wave owns 32*NQ of them and consumes every tile ("row split").  When no more
-// than 32*NQ rows are left the four waves instead share those rows and each consumes one of the
-// four tiles of a super tile ("token split"); their states are merged at the end.
-template <typename E, int D, int NQ, bool GATHERED>
-__global__ void __launch_bounds__(kBlock) stage1_dense_kernel(Stage1Args a) {
+// One block (8 waves) per (vnode, kv head).  The block streams the vnode's KV run through LDS
+// 128 tokens at a time with direct global->LDS loads; the next super tile is in flight while
+// the current one is consumed.  Per pass over the run the waves form RG row groups of 32 query
+// rows x TG token groups (RG * TG = 8, or 4 when only 32 rows are left): a wave consumes the
+// tiles tg, tg + TG, .. of every super tile for the rows of its row group, and the TG states of
+// a row group are merged at the end.
+template <typename E, int D, bool GATHERED>
+__global__ void __launch_bounds__(kWideBlock) stage1_dense_kernel(Stage1Args a) {
   using W = WideGeom<D>;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -700,7 +724,6 @@ __global__ void __launch_bounds__(kBlock) stage1_dense_kernel(Stage1Args a) {
   const VnodeView vn = load_vnode<GATHERED>(a, a.vnode_begin + blockIdx.x);
   const int rows_total = vn.q_len * a.g;
   const int nsuper = (vn.kv_len + W::kTokens - 1) / W::kTokens;
-  constexpr int kWaveRows = 32 * NQ;
 
   // loader role of this lane: 16-byte slot `pos` of row `grp_row` in each 1 KB group it fills
   const int grp_row = lane / W::kChunks, pos = lane % W::kChunks;
@@ -708,21 +731,26 @@ __global__ void __launch_bounds__(kBlock) stage1_dense_kernel(Stage1Args a) {
   const char* vbase = a.v + 2 * ((int64_t)kvh * a.sv1);
 
   for (int row0 = 0; row0 < rows_total;) {
-    const bool token_split = rows_total - row0 <= kWaveRows;
-    const int my_row0 = token_split ? row0 : row0 + wave * kWaveRows;
-    const bool has_rows = my_row0 < rows_total;
+    const int groups = (rows_total - row0 + 31) >> 5;   // 32-row groups still to serve
+    const int tgroups = groups >= 5 ? 1 : (groups >= 3 ? 2 : 4);
+    const int rgroups = groups >= 5 ? 8 : (groups >= 3 ? 4 : (groups == 2 ? 2 : 1));
+    const int rg = wave / tgroups, tg = wave % tgroups;
+    const int my_row0 = row0 + 32 * rg;
+    const bool active = rg < rgroups && my_row0 < rows_total;
 
-    u32x4 qf[NQ][D / 16];
-    load_q_frags32<D, NQ, GATHERED>(a, vn, kvh, my_row0, qf);
-    WideState<D, NQ> st;
-    reset_state<D, NQ>(st);
+    u32x4 qf[D / 16];
+    load_q_frags32<D, GATHERED>(a, vn, kvh, active ? my_row0 : rows_total, qf);
+    WideState<D> st;
+    reset_state<D>(st);
+    WideLane la;
+    init_lane<D>(la);
 
-    // slots of the rows this lane loads in the next super tile (group g = j*4 + wave)
+    // slots of the rows this lane loads in the next super tile (group g = j*8 + wave)
     int slot[W::kGroupsPerWave];
     auto load_slots = [&](int super) {
 #pragma unroll
       for (int j = 0; j < W::kGroupsPerWave; ++j) {
-        const int t = super * W::kTokens + (j * kWavesPerBlock + wave) * W::kGroupRows + grp_row;
+        const int t = super * W::kTokens + (j * kWideWaves + wave) * W::kGroupRows + grp_row;
         slot[j] = -1;
         if (t < vn.kv_len) slot[j] = GATHERED ? (int)t : a.kv_entries[vn.kv_base + t];
       }
@@ -732,7 +760,7 @@ __global__ void __launch_bounds__(kBlock) stage1_dense_kernel(Stage1Args a) {
       char* bufV = bufK + W::kBytesK;
 #pragma unroll
       for (int j = 0; j < W::kGroupsPerWave; ++j) {
-        const int grp = j * kWavesPerBlock + wave;
+        const int grp = j * kWideWaves + wave;
         const int row = grp * W::kGroupRows + grp_row;
         const int chunk = pos ^ W::swz(row);
         char* dstK = bufK + grp * 1024;   // wave-uniform; lane l lands at +16*l
@@ -754,42 +782,44 @@ __global__ void __launch_bounds__(kBlock) stage1_dense_kernel(Stage1Args a) {
       issue_rows(0);
       if (nsuper > 1) load_slots(1);
     }
+    FT_TIME(unsigned long long t_start = FT_CLOCK(); unsigned long long t_wait = 0, t_bar = 0, t_issue = 0, t_comp = 0;)
     for (int super = 0; super < nsuper; ++super) {
       // the loads of this super tile were issued one iteration ago; publish them to the block
+      FT_TIME(unsigned long long c0 = FT_CLOCK();)
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      FT_TIME(unsigned long long c1 = FT_CLOCK();)
       __syncthreads();
+      FT_TIME(unsigned long long c2 = FT_CLOCK();)
       // the other buffer was last read before that barrier: refill it now
       if (super + 1 < nsuper) {
         issue_rows(super + 1);
         if (super + 2 < nsuper) load_slots(super + 2);
       }
-      const char* bufK = smem + (super & 1) * W::kBytes;
-      const char* bufV = bufK + W::kBytesK;
-      if (has_rows) {
+      FT_TIME(unsigned long long c3 = FT_CLOCK();)
+      if (active) {
         const int left = vn.kv_len - super * W::kTokens;  // tokens from the start of this super tile
-        if (token_split) {
-          const int valid = left - wave * kTileTokens;
-          if (valid > 0)
-            tile_step32<E, D, NQ>(bufK + wave * W::kTileBytes, bufV + wave * W::kTileBytes, valid, a.scale_log2, qf, st);
-        } else {
 #pragma unroll 1
-          for (int sub = 0; sub < W::kSub; ++sub) {
-            const int valid = left - sub * kTileTokens;
-            if (valid > 0)
-              tile_step32<E, D, NQ>(bufK + sub * W::kTileBytes, bufV + sub * W::kTileBytes, valid, a.scale_log2, qf, st);
-          }
+        for (int sub = tg; sub < W::kSub; sub += tgroups) {
+          const int valid = left - sub * kTileTokens;
+          if (valid >= kTileTokens)
+            tile_step32<E, D, false>(la, sub * W::kTileBytes, valid, a.scale_log2, qf, st);
+          else if (valid > 0)
+            tile_step32<E, D, true>(la, sub * W::kTileBytes, valid, a.scale_log2, qf, st);
         }
       }
+      flip_buffer<D>(la);
+      FT_TIME(unsigned long long c4 = FT_CLOCK(); t_wait += c1 - c0; t_bar += c2 - c1; t_issue += c3 - c2; t_comp += c4 - c3;)
     }
-    finish_state<D, NQ>(st);
-    if (token_split) {
-      merge_waves<D, NQ>(reinterpret_cast<float*>(smem), st);
-      if (wave == 0) write_partials32<D, NQ>(a, vn, kvh, my_row0, st);
-    } else if (has_rows) {
-      write_partials32<D, NQ>(a, vn, kvh, my_row0, st);
-    }
+    FT_TIME(if (g_timing && lane == 0) {
+      unsigned long long* out = g_timing + ((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * kWideWaves + wave) * 8;
+      out[0] = t_wait; out[1] = t_bar; out[2] = t_issue; out[3] = t_comp; out[4] = FT_CLOCK() - t_start; out[5] = nsuper;
+      out[6] = t_start; out[7] = 0;
+    })
+    finish_state<D>(st);
+    if (tgroups > 1) merge_token_groups<D>(reinterpret_cast<float*>(smem), st, rg, tg, tgroups, active);
+    if (active && tg == 0) write_partials32<D>(a, vn, kvh, my_row0, st);
     __syncthreads();  // staging LDS is reused by the next pass over the run
-    row0 += token_split ? kWaveRows : kWavesPerBlock * kWaveRows;
+    row0 += 32 * rgroups;
   }
 }
 
@@ -890,10 +920,10 @@ int launch_stage1_inst(const Stage1Args& a, int hkv, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? FT_OK : FT_ERR_LAUNCH;
 }
 
-template <typename E, int D, int NQ, bool GATHERED>
+template <typename E, int D, bool GATHERED>
 int launch_stage1_dense(const Stage1Args& a, int hkv, hipStream_t stream) {
   const size_t lds = 2 * (size_t)WideGeom<D>::kBytes;
-  auto kern = stage1_dense_kernel<E, D, NQ, GATHERED>;
+  auto kern = stage1_dense_kernel<E, D, GATHERED>;
   static bool configured = false;
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
@@ -902,21 +932,19 @@ int launch_stage1_dense(const Stage1Args& a, int hkv, hipStream_t stream) {
     }
     configured = true;
   }
-  hipLaunchKernelGGL(kern, dim3((unsigned)a.vnode_count, (unsigned)hkv, 1), dim3(kBlock, 1, 1), lds, stream, a);
+  hipLaunchKernelGGL(kern, dim3((unsigned)a.vnode_count, (unsigned)hkv, 1), dim3(kWideBlock, 1, 1), lds, stream, a);
   return hipGetLastError() == hipSuccess ? FT_OK : FT_ERR_LAUNCH;
 }
 
 template <typename E, int D, bool GATHERED>
 int launch_stage1_d(const Stage1Args& a, int hkv, int rows_per_vnode, hipStream_t stream) {
-  // Narrow vnodes (<= 16 rows): one wave each.  Wider: one block each, 32 or 64 rows per wave
-  // and up to four waves' worth of rows per pass over the KV run.
+  // Narrow vnodes (<= 16 rows): one wave each.  Wider: one 8-wave block each.
   if (rows_per_vnode <= 16) return launch_stage1_inst<E, D, 1, false, GATHERED>(a, hkv, stream);
   if constexpr (D > 128) {
-    // 128-token double buffers of 256-wide rows do not fit in LDS: per-wave staging instead
+    // 128-token double buffers of 512-byte rows do not fit in LDS: per-wave staging instead
     return launch_stage1_inst<E, D, 2, true, GATHERED>(a, hkv, stream);
   } else {
-    if (rows_per_vnode <= 32) return launch_stage1_dense<E, D, 1, GATHERED>(a, hkv, stream);
-    return launch_stage1_dense<E, D, 2, GATHERED>(a, hkv, stream);
+    return launch_stage1_dense<E, D, GATHERED>(a, hkv, stream);
   }
 }
 
@@ -967,6 +995,12 @@ int check_common(int d, int g, int dtype) {
 }
 
 }  // namespace
+
+#ifdef FT_TIMING
+extern "C" int ft_debug_set_timing(unsigned long long* buf) {
+  return hipMemcpyToSymbol(HIP_SYMBOL(g_timing), &buf, sizeof(buf)) == hipSuccess ? 0 : -1;
+}
+#endif
 
 extern "C" {
 
