@@ -117,6 +117,7 @@ struct Stage1Args {
   const int32_t* q_lens;
   int vnode_begin, vnode_count;
   int g;
+  int hkv;
   float scale_log2;  // sm_scale * log2(e)
   float* mid_o;
   int64_t so0, so1;
@@ -594,6 +595,9 @@ __device__ __forceinline__ void tile_step32(const WideLane& la, unsigned off, in
   u32x4 kf[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) kf[ks] = lds_read16(kb ^ (32u * ks));
+  // (keeps the scheduler from sinking each read next to its use, which would expose the full
+  // LDS latency eight times in a row)
+  __builtin_amdgcn_sched_barrier(0);
   f32x16 s;
 #pragma unroll
   for (int j = 0; j < 16; ++j) s[j] = 0.f;
@@ -720,8 +724,12 @@ __global__ void __launch_bounds__(kWideBlock) stage1_dense_kernel(Stage1Args a) 
   using W = WideGeom<D>;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int kvh = blockIdx.y;
-  const VnodeView vn = load_vnode<GATHERED>(a, a.vnode_begin + blockIdx.x);
+  // The KV head varies fastest over the (1-D) grid: blocks are handed to the 8 XCDs round robin,
+  // so with 8 KV heads every head's KV stays in one XCD's L2, and the vnodes of a phase are
+  // started in list order (the planner lists the widest, longest ones first).
+  const int local_vnode = blockIdx.x / a.hkv;
+  const int kvh = blockIdx.x - local_vnode * a.hkv;
+  const VnodeView vn = load_vnode<GATHERED>(a, a.vnode_begin + local_vnode);
   const int rows_total = vn.q_len * a.g;
   const int nsuper = (vn.kv_len + W::kTokens - 1) / W::kTokens;
 
@@ -782,7 +790,7 @@ __global__ void __launch_bounds__(kWideBlock) stage1_dense_kernel(Stage1Args a) 
       issue_rows(0);
       if (nsuper > 1) load_slots(1);
     }
-    FT_TIME(unsigned long long t_start = FT_CLOCK(); unsigned long long t_wait = 0, t_bar = 0, t_issue = 0, t_comp = 0;)
+    FT_TIME(unsigned long long t_start = FT_CLOCK(); unsigned long long rt_start = wall_clock64(); unsigned long long t_wait = 0, t_bar = 0, t_issue = 0, t_comp = 0;)
     for (int super = 0; super < nsuper; ++super) {
       // the loads of this super tile were issued one iteration ago; publish them to the block
       FT_TIME(unsigned long long c0 = FT_CLOCK();)
@@ -811,9 +819,9 @@ __global__ void __launch_bounds__(kWideBlock) stage1_dense_kernel(Stage1Args a) 
       FT_TIME(unsigned long long c4 = FT_CLOCK(); t_wait += c1 - c0; t_bar += c2 - c1; t_issue += c3 - c2; t_comp += c4 - c3;)
     }
     FT_TIME(if (g_timing && lane == 0) {
-      unsigned long long* out = g_timing + ((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * kWideWaves + wave) * 8;
+      unsigned long long* out = g_timing + ((size_t)blockIdx.x * kWideWaves + wave) * 8;
       out[0] = t_wait; out[1] = t_bar; out[2] = t_issue; out[3] = t_comp; out[4] = FT_CLOCK() - t_start; out[5] = nsuper;
-      out[6] = t_start; out[7] = 0;
+      out[6] = rt_start; out[7] = wall_clock64();
     })
     finish_state<D>(st);
     if (tgroups > 1) merge_token_groups<D>(reinterpret_cast<float*>(smem), st, rg, tg, tgroups, active);
@@ -932,7 +940,7 @@ int launch_stage1_dense(const Stage1Args& a, int hkv, hipStream_t stream) {
     }
     configured = true;
   }
-  hipLaunchKernelGGL(kern, dim3((unsigned)a.vnode_count, (unsigned)hkv, 1), dim3(kWideBlock, 1, 1), lds, stream, a);
+  hipLaunchKernelGGL(kern, dim3((unsigned)((int64_t)hkv * a.vnode_count), 1, 1), dim3(kWideBlock, 1, 1), lds, stream, a);
   return hipGetLastError() == hipSuccess ? FT_OK : FT_ERR_LAUNCH;
 }
 
@@ -1035,7 +1043,8 @@ int ft_stage1(const void* q, const void* k, const void* v,
   if (!q || !k || !v || !vnode_to_kv_entries || !vnode_to_kv_offs || !vnode_to_kv_lens || !vnode_to_q_entries ||
       !vnode_to_q_offs || !vnode_to_q_lens || !mid_o || !mid_lse)
     return FT_ERR_NULL_POINTER;
-  if (vnode_begin < 0 || vnode_count < 0 || num_kv_heads < 1 || num_kv_heads > 65535 || q_tile < 1 || !(sm_scale > 0.f))
+  if (vnode_begin < 0 || vnode_count < 0 || num_kv_heads < 1 || num_kv_heads > 65535 || q_tile < 1 || !(sm_scale > 0.f) ||
+      (int64_t)vnode_count * num_kv_heads > INT32_MAX)
     return FT_ERR_ARGUMENT;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(mid_o) || (sq0 | sq1 | sk0 | sk1 | sv0 | sv1) % 8 != 0 ||
       (so0 | so1) % 4 != 0)
@@ -1049,6 +1058,7 @@ int ft_stage1(const void* q, const void* k, const void* v,
   a.q_entries = vnode_to_q_entries; a.q_offs = vnode_to_q_offs; a.q_lens = vnode_to_q_lens;
   a.vnode_begin = vnode_begin; a.vnode_count = vnode_count;
   a.g = kv_group_num;
+  a.hkv = num_kv_heads;
   a.scale_log2 = sm_scale * kLog2e;
   a.mid_o = mid_o; a.so0 = so0; a.so1 = so1; a.mid_lse = mid_lse; a.sl0 = sl0;
   const int64_t rows = (int64_t)q_tile * kv_group_num;
@@ -1129,6 +1139,7 @@ int ft_gathered_decode(const void* q, const void* k_cache, const void* v_cache,
   a.sk1 = a.sv1 = head_dim;
   a.vnode_begin = 0; a.vnode_count = batch_size * nsplit;
   a.g = g;
+  a.hkv = num_kv_heads;
   a.scale_log2 = sm_scale * kLog2e;
   a.mid_o = mid_o; a.so0 = (int64_t)num_qo_heads * head_dim; a.so1 = head_dim;
   a.mid_lse = mid_lse; a.sl0 = num_qo_heads;
