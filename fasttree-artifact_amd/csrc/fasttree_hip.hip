@@ -115,7 +115,8 @@ struct Stage1Args {
   const int32_t* q_entries;
   const int32_t* q_offs;
   const int32_t* q_lens;
-  int vnode_begin, vnode_count;
+  int vnode_begin, vnode_count;    // vnodes served by 8-wave blocks (or the whole range for the per-wave-staging kernel)
+  int narrow_begin, narrow_count;  // vnodes of at most 16 rows, served by one wave each
   int g;
   int hkv;
   float scale_log2;  // sm_scale * log2(e)
@@ -720,15 +721,9 @@ __device__ __forceinline__ void merge_token_groups(float* xchg, WideState<D>& st
 // tiles tg, tg + TG, .. of every super tile for the rows of its row group, and the TG states of
 // a row group are merged at the end.
 template <typename E, int D, bool GATHERED>
-__global__ void __launch_bounds__(kWideBlock) stage1_dense_kernel(Stage1Args a) {
+__device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int local_vnode, int kvh) {
   using W = WideGeom<D>;
-  extern __shared__ __attribute__((aligned(16))) char smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  // The KV head varies fastest over the (1-D) grid: blocks are handed to the 8 XCDs round robin,
-  // so with 8 KV heads every head's KV stays in one XCD's L2, and the vnodes of a phase are
-  // started in list order (the planner lists the widest, longest ones first).
-  const int local_vnode = blockIdx.x / a.hkv;
-  const int kvh = blockIdx.x - local_vnode * a.hkv;
   const VnodeView vn = load_vnode<GATHERED>(a, a.vnode_begin + local_vnode);
   const int rows_total = vn.q_len * a.g;
   const int nsuper = (vn.kv_len + W::kTokens - 1) / W::kTokens;
@@ -819,7 +814,7 @@ __global__ void __launch_bounds__(kWideBlock) stage1_dense_kernel(Stage1Args a) 
       FT_TIME(unsigned long long c4 = FT_CLOCK(); t_wait += c1 - c0; t_bar += c2 - c1; t_issue += c3 - c2; t_comp += c4 - c3;)
     }
     FT_TIME(if (g_timing && lane == 0) {
-      unsigned long long* out = g_timing + ((size_t)blockIdx.x * kWideWaves + wave) * 8;
+      unsigned long long* out = g_timing + ((size_t)(local_vnode * a.hkv + kvh) * kWideWaves + wave) * 8;
       out[0] = t_wait; out[1] = t_bar; out[2] = t_issue; out[3] = t_comp; out[4] = FT_CLOCK() - t_start; out[5] = nsuper;
       out[6] = rt_start; out[7] = wall_clock64();
     })
@@ -828,6 +823,36 @@ __global__ void __launch_bounds__(kWideBlock) stage1_dense_kernel(Stage1Args a) 
     if (active && tg == 0) write_partials32<D>(a, vn, kvh, my_row0, st);
     __syncthreads();  // staging LDS is reused by the next pass over the run
     row0 += 32 * rgroups;
+  }
+}
+
+// Stage 1 in one launch.  Blocks [0, wide vnodes x KV heads) serve the wide vnodes, one block
+// per (vnode, KV head); the blocks after them serve the narrow vnodes, one wave per (vnode, KV
+// head).  The KV head varies fastest: blocks are handed to the 8 XCDs round robin, so with 8 KV
+// heads every head's KV stays in one XCD's L2.  The wide vnodes start first, in list order (the
+// planner lists the widest, longest ones first); the many short narrow items then fill the
+// compute units as the wide blocks drain, and their HBM-bound streaming overlaps the
+// matrix-bound tail.
+template <typename E, int D, bool GATHERED>
+__global__ void __launch_bounds__(kWideBlock) stage1_fused_kernel(Stage1Args a) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int wide_blocks = a.vnode_count * a.hkv;
+  if ((int)blockIdx.x < wide_blocks) {
+    const int local_vnode = blockIdx.x / a.hkv;
+    wide_block<E, D, GATHERED>(a, smem, local_vnode, blockIdx.x - local_vnode * a.hkv);
+  } else {
+    const int wave = threadIdx.x >> 6;
+    const int item = (blockIdx.x - wide_blocks) * kWideWaves + wave;
+    if (item >= a.narrow_count * a.hkv) return;  // whole wave; no block barrier below
+    const int local_vnode = item / a.hkv;
+    const int kvh = item - local_vnode * a.hkv;
+    const VnodeView vn = load_vnode<GATHERED>(a, a.narrow_begin + local_vnode);
+    const int rows_total = vn.q_len * a.g;
+    for (int row0 = 0; row0 < rows_total; row0 += 16) {
+      WaveState<D, 1> st;
+      wave_attend<E, D, 1, GATHERED>(a, vn, kvh, row0, 0, 1, smem + wave * TileGeom<D>::kBytes, st);
+      write_partials<D, 1>(a, vn, kvh, row0, st);
+    }
   }
 }
 
@@ -929,10 +954,12 @@ int launch_stage1_inst(const Stage1Args& a, int hkv, hipStream_t stream) {
 }
 
 template <typename E, int D, bool GATHERED>
-int launch_stage1_dense(const Stage1Args& a, int hkv, hipStream_t stream) {
-  const size_t lds = 2 * (size_t)WideGeom<D>::kBytes;
-  auto kern = stage1_dense_kernel<E, D, GATHERED>;
-  static bool configured = false;
+int launch_stage1_fused(const Stage1Args& a, hipStream_t stream) {
+  constexpr size_t kWideLds = 2 * (size_t)WideGeom<D>::kBytes;
+  constexpr size_t kNarrowLds = (size_t)kWideWaves * TileGeom<D>::kBytes;
+  constexpr size_t lds = kWideLds > kNarrowLds ? kWideLds : kNarrowLds;
+  auto kern = stage1_fused_kernel<E, D, GATHERED>;
+  static bool configured = false;  // raising the dynamic LDS limit is idempotent
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
       (void)hipGetLastError();
@@ -940,31 +967,43 @@ int launch_stage1_dense(const Stage1Args& a, int hkv, hipStream_t stream) {
     }
     configured = true;
   }
-  hipLaunchKernelGGL(kern, dim3((unsigned)((int64_t)hkv * a.vnode_count), 1, 1), dim3(kWideBlock, 1, 1), lds, stream, a);
+  const int64_t narrow_items = (int64_t)a.narrow_count * a.hkv;
+  const int64_t blocks = (int64_t)a.vnode_count * a.hkv + (narrow_items + kWideWaves - 1) / kWideWaves;
+  if (blocks == 0) return FT_OK;
+  if (blocks > INT32_MAX) return FT_ERR_ARGUMENT;
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks, 1, 1), dim3(kWideBlock, 1, 1), lds, stream, a);
   return hipGetLastError() == hipSuccess ? FT_OK : FT_ERR_LAUNCH;
 }
 
+// `a` names two vnode ranges: [vnode_begin, +vnode_count) of wide vnodes (more than 16 query
+// rows) and [narrow_begin, +narrow_count) of narrow ones.
 template <typename E, int D, bool GATHERED>
-int launch_stage1_d(const Stage1Args& a, int hkv, int rows_per_vnode, hipStream_t stream) {
-  // Narrow vnodes (<= 16 rows): one wave each.  Wider: one 8-wave block each.
-  if (rows_per_vnode <= 16) return launch_stage1_inst<E, D, 1, false, GATHERED>(a, hkv, stream);
+int launch_stage1_d(const Stage1Args& a, hipStream_t stream) {
   if constexpr (D > 128) {
-    // 128-token double buffers of 512-byte rows do not fit in LDS: per-wave staging instead
-    return launch_stage1_inst<E, D, 2, true, GATHERED>(a, hkv, stream);
+    // 128-token double buffers of 512-byte rows do not fit in LDS: per-wave staging kernels
+    if (a.vnode_count > 0)
+      if (int rc = launch_stage1_inst<E, D, 2, true, GATHERED>(a, a.hkv, stream)) return rc;
+    if (a.narrow_count > 0) {
+      Stage1Args n = a;
+      n.vnode_begin = a.narrow_begin;
+      n.vnode_count = a.narrow_count;
+      return launch_stage1_inst<E, D, 1, false, GATHERED>(n, a.hkv, stream);
+    }
+    return FT_OK;
   } else {
-    return launch_stage1_dense<E, D, GATHERED>(a, hkv, stream);
+    return launch_stage1_fused<E, D, GATHERED>(a, stream);
   }
 }
 
 template <bool GATHERED>
-int launch_stage1(const Stage1Args& a, int hkv, int d, int rows_per_vnode, int dtype, hipStream_t stream) {
-#define FT_DISPATCH_D(E)                                                                  \
-  switch (d) {                                                                            \
-    case 32: return launch_stage1_d<E, 32, GATHERED>(a, hkv, rows_per_vnode, stream);     \
-    case 64: return launch_stage1_d<E, 64, GATHERED>(a, hkv, rows_per_vnode, stream);     \
-    case 128: return launch_stage1_d<E, 128, GATHERED>(a, hkv, rows_per_vnode, stream);   \
-    case 256: return launch_stage1_d<E, 256, GATHERED>(a, hkv, rows_per_vnode, stream);   \
-    default: return FT_ERR_HEAD_DIM;                                                      \
+int launch_stage1(const Stage1Args& a, int d, int dtype, hipStream_t stream) {
+#define FT_DISPATCH_D(E)                                              \
+  switch (d) {                                                        \
+    case 32: return launch_stage1_d<E, 32, GATHERED>(a, stream);      \
+    case 64: return launch_stage1_d<E, 64, GATHERED>(a, stream);      \
+    case 128: return launch_stage1_d<E, 128, GATHERED>(a, stream);    \
+    case 256: return launch_stage1_d<E, 256, GATHERED>(a, stream);    \
+    default: return FT_ERR_HEAD_DIM;                                  \
   }
   if (dtype == FT_DTYPE_F16) { FT_DISPATCH_D(F16) }
   if (dtype == FT_DTYPE_BF16) { FT_DISPATCH_D(BF16) }
@@ -1028,6 +1067,44 @@ const char* ft_error_string(int code) {
   }
 }
 
+// Validates the stage-1 arguments shared by ft_stage1 and ft_decode and fills everything of
+// `a` but the vnode ranges.
+static int stage1_setup(Stage1Args& a, const void* q, const void* k, const void* v,
+                        int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+                        const int32_t* vnode_to_kv_entries, const int32_t* vnode_to_kv_offs,
+                        const int32_t* vnode_to_kv_lens, const int32_t* vnode_to_q_entries,
+                        const int32_t* vnode_to_q_offs, const int32_t* vnode_to_q_lens,
+                        int num_kv_heads, int kv_group_num, int head_dim, float sm_scale,
+                        float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0, int dtype) {
+  if (int rc = check_common(head_dim, kv_group_num, dtype)) return rc;
+  if (!q || !k || !v || !vnode_to_kv_entries || !vnode_to_kv_offs || !vnode_to_kv_lens || !vnode_to_q_entries ||
+      !vnode_to_q_offs || !vnode_to_q_lens || !mid_o || !mid_lse)
+    return FT_ERR_NULL_POINTER;
+  if (num_kv_heads < 1 || num_kv_heads > 65535 || !(sm_scale > 0.f)) return FT_ERR_ARGUMENT;
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(mid_o) || (sq0 | sq1 | sk0 | sk1 | sv0 | sv1) % 8 != 0 ||
+      (so0 | so1) % 4 != 0)
+    return FT_ERR_ALIGNMENT;
+  a = Stage1Args{};
+  a.q = static_cast<const char*>(q);
+  a.k = static_cast<const char*>(k);
+  a.v = static_cast<const char*>(v);
+  a.sq0 = sq0; a.sq1 = sq1; a.sk0 = sk0; a.sk1 = sk1; a.sv0 = sv0; a.sv1 = sv1;
+  a.kv_entries = vnode_to_kv_entries; a.kv_offs = vnode_to_kv_offs; a.kv_lens = vnode_to_kv_lens;
+  a.q_entries = vnode_to_q_entries; a.q_offs = vnode_to_q_offs; a.q_lens = vnode_to_q_lens;
+  a.g = kv_group_num;
+  a.hkv = num_kv_heads;
+  a.scale_log2 = sm_scale * kLog2e;
+  a.mid_o = mid_o; a.so0 = so0; a.so1 = so1; a.mid_lse = mid_lse; a.sl0 = sl0;
+  return FT_OK;
+}
+
+// A phase whose tile holds at most 16 query rows is served one wave per (vnode, KV head).
+static bool is_narrow(int q_tile, int kv_group_num) { return (int64_t)q_tile * kv_group_num <= 16; }
+
+static bool range_ok(int begin, int count, int num_kv_heads) {
+  return begin >= 0 && count >= 0 && (int64_t)count * num_kv_heads <= INT32_MAX;
+}
+
 int ft_stage1(const void* q, const void* k, const void* v,
               int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
               const int32_t* vnode_to_kv_entries, const int32_t* vnode_to_kv_offs,
@@ -1040,29 +1117,18 @@ int ft_stage1(const void* q, const void* k, const void* v,
   (void)kv_tile;
   if (int rc = check_common(head_dim, kv_group_num, dtype)) return rc;
   if (vnode_count == 0) return FT_OK;
-  if (!q || !k || !v || !vnode_to_kv_entries || !vnode_to_kv_offs || !vnode_to_kv_lens || !vnode_to_q_entries ||
-      !vnode_to_q_offs || !vnode_to_q_lens || !mid_o || !mid_lse)
-    return FT_ERR_NULL_POINTER;
-  if (vnode_begin < 0 || vnode_count < 0 || num_kv_heads < 1 || num_kv_heads > 65535 || q_tile < 1 || !(sm_scale > 0.f) ||
-      (int64_t)vnode_count * num_kv_heads > INT32_MAX)
-    return FT_ERR_ARGUMENT;
-  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(mid_o) || (sq0 | sq1 | sk0 | sk1 | sv0 | sv1) % 8 != 0 ||
-      (so0 | so1) % 4 != 0)
-    return FT_ERR_ALIGNMENT;
-  Stage1Args a{};
-  a.q = static_cast<const char*>(q);
-  a.k = static_cast<const char*>(k);
-  a.v = static_cast<const char*>(v);
-  a.sq0 = sq0; a.sq1 = sq1; a.sk0 = sk0; a.sk1 = sk1; a.sv0 = sv0; a.sv1 = sv1;
-  a.kv_entries = vnode_to_kv_entries; a.kv_offs = vnode_to_kv_offs; a.kv_lens = vnode_to_kv_lens;
-  a.q_entries = vnode_to_q_entries; a.q_offs = vnode_to_q_offs; a.q_lens = vnode_to_q_lens;
-  a.vnode_begin = vnode_begin; a.vnode_count = vnode_count;
-  a.g = kv_group_num;
-  a.hkv = num_kv_heads;
-  a.scale_log2 = sm_scale * kLog2e;
-  a.mid_o = mid_o; a.so0 = so0; a.so1 = so1; a.mid_lse = mid_lse; a.sl0 = sl0;
-  const int64_t rows = (int64_t)q_tile * kv_group_num;
-  return launch_stage1<false>(a, num_kv_heads, head_dim, rows > 64 ? 64 : (int)rows, dtype, stream);
+  Stage1Args a;
+  if (int rc = stage1_setup(a, q, k, v, sq0, sq1, sk0, sk1, sv0, sv1, vnode_to_kv_entries, vnode_to_kv_offs,
+                            vnode_to_kv_lens, vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, num_kv_heads,
+                            kv_group_num, head_dim, sm_scale, mid_o, so0, so1, mid_lse, sl0, dtype))
+    return rc;
+  if (q_tile < 1 || !range_ok(vnode_begin, vnode_count, num_kv_heads)) return FT_ERR_ARGUMENT;
+  if (is_narrow(q_tile, kv_group_num)) {
+    a.narrow_begin = vnode_begin; a.narrow_count = vnode_count;
+  } else {
+    a.vnode_begin = vnode_begin; a.vnode_count = vnode_count;
+  }
+  return launch_stage1<false>(a, head_dim, dtype, stream);
 }
 
 int ft_stage2(const int32_t* req_to_vnode_entries, const int32_t* req_to_vnode_offs,
@@ -1084,6 +1150,56 @@ int ft_stage2(const int32_t* req_to_vnode_entries, const int32_t* req_to_vnode_o
   return launch_stage2(a, head_dim, dtype, stream);
 }
 
+int ft_stage1_phases(const void* q, const void* k, const void* v,
+                     int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+                     const int32_t* vnode_to_kv_entries, const int32_t* vnode_to_kv_offs,
+                     const int32_t* vnode_to_kv_lens, const int32_t* vnode_to_q_entries,
+                     const int32_t* vnode_to_q_offs, const int32_t* vnode_to_q_lens,
+                     float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
+                     const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
+                     const int32_t phase_q_tile_sizes[2], const int32_t phase_kv_tile_sizes[2],
+                     int num_qo_heads, int num_kv_heads, int head_dim,
+                     float sm_scale, int dtype, ft_stream_t stream) {
+  if (!phase_node_nums || !phase_node_offsets || !phase_q_tile_sizes || !phase_kv_tile_sizes) return FT_ERR_NULL_POINTER;
+  if (num_kv_heads < 1 || num_qo_heads % num_kv_heads != 0) return FT_ERR_GROUP;
+  const int g = num_qo_heads / num_kv_heads;
+  if (int rc = check_common(head_dim, g, dtype)) return rc;
+  if (phase_node_nums[0] == 0 && phase_node_nums[1] == 0) return FT_OK;
+  Stage1Args a;
+  if (int rc = stage1_setup(a, q, k, v, sq0, sq1, sk0, sk1, sv0, sv1, vnode_to_kv_entries, vnode_to_kv_offs,
+                            vnode_to_kv_lens, vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, num_kv_heads, g,
+                            head_dim, sm_scale, mid_o, so0, so1, mid_lse, sl0, dtype))
+    return rc;
+  const bool pending[2] = {phase_node_nums[0] != 0, phase_node_nums[1] != 0};
+  for (int phase = 0; phase < 2; ++phase)
+    if (pending[phase] && (phase_q_tile_sizes[phase] < 1 ||
+                           !range_ok(phase_node_offsets[phase], phase_node_nums[phase], num_kv_heads)))
+      return FT_ERR_ARGUMENT;
+  const bool narrow[2] = {is_narrow(phase_q_tile_sizes[0], g), is_narrow(phase_q_tile_sizes[1], g)};
+  auto assign = [](Stage1Args& t, bool is_narrow_range, int begin, int count) {
+    if (is_narrow_range) { t.narrow_begin = begin; t.narrow_count = count; }
+    else { t.vnode_begin = begin; t.vnode_count = count; }
+  };
+  // Both phases go into one launch when one is wide and the other narrow, or when they are of
+  // the same kind and adjacent in the vnode list (the planner's lists always are).
+  if (pending[0] && pending[1] && narrow[0] == narrow[1]) {
+    if (phase_node_offsets[0] + phase_node_nums[0] == phase_node_offsets[1] &&
+        range_ok(phase_node_offsets[0], phase_node_nums[0] + phase_node_nums[1], num_kv_heads)) {
+      assign(a, narrow[0], phase_node_offsets[0], phase_node_nums[0] + phase_node_nums[1]);
+      return launch_stage1<false>(a, head_dim, dtype, stream);
+    }
+    for (int phase = 0; phase < 2; ++phase) {
+      Stage1Args b = a;
+      assign(b, narrow[phase], phase_node_offsets[phase], phase_node_nums[phase]);
+      if (int rc = launch_stage1<false>(b, head_dim, dtype, stream)) return rc;
+    }
+    return FT_OK;
+  }
+  for (int phase = 0; phase < 2; ++phase)
+    if (pending[phase]) assign(a, narrow[phase], phase_node_offsets[phase], phase_node_nums[phase]);
+  return launch_stage1<false>(a, head_dim, dtype, stream);
+}
+
 int ft_decode(const void* q, const void* k, const void* v, void* o,
               int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
               int64_t oo0, int64_t oo1,
@@ -1097,18 +1213,11 @@ int ft_decode(const void* q, const void* k, const void* v, void* o,
               const int32_t phase_q_tile_sizes[2], const int32_t phase_kv_tile_sizes[2],
               int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
               float sm_scale, int dtype, ft_stream_t stream) {
-  if (!phase_node_nums || !phase_node_offsets || !phase_q_tile_sizes || !phase_kv_tile_sizes) return FT_ERR_NULL_POINTER;
-  if (num_kv_heads < 1 || num_qo_heads % num_kv_heads != 0) return FT_ERR_GROUP;
-  const int g = num_qo_heads / num_kv_heads;
-  for (int phase = 0; phase < 2; ++phase) {
-    if (phase_node_nums[phase] == 0) continue;
-    if (int rc = ft_stage1(q, k, v, sq0, sq1, sk0, sk1, sv0, sv1, vnode_to_kv_entries, vnode_to_kv_offs,
-                           vnode_to_kv_lens, vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens,
-                           phase_node_offsets[phase], phase_node_nums[phase], num_kv_heads, g, head_dim,
-                           phase_q_tile_sizes[phase], phase_kv_tile_sizes[phase], sm_scale, mid_o, so0, so1,
-                           mid_lse, sl0, dtype, stream))
-      return rc;
-  }
+  if (int rc = ft_stage1_phases(q, k, v, sq0, sq1, sk0, sk1, sv0, sv1, vnode_to_kv_entries, vnode_to_kv_offs,
+                                vnode_to_kv_lens, vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, mid_o, so0, so1,
+                                mid_lse, sl0, phase_node_nums, phase_node_offsets, phase_q_tile_sizes,
+                                phase_kv_tile_sizes, num_qo_heads, num_kv_heads, head_dim, sm_scale, dtype, stream))
+    return rc;
   return ft_stage2(req_to_vnode_entries, req_to_vnode_offs, req_to_vnode_lens, mid_o, so0, so1, mid_lse, sl0, o, oo0,
                    oo1, batch_size, num_qo_heads, head_dim, dtype, stream);
 }
@@ -1137,14 +1246,15 @@ int ft_gathered_decode(const void* q, const void* k_cache, const void* v_cache,
   a.sq0 = sq0; a.sq1 = sq1;
   a.sk0 = a.sv0 = (int64_t)num_kv_heads * head_dim;
   a.sk1 = a.sv1 = head_dim;
-  a.vnode_begin = 0; a.vnode_count = batch_size * nsplit;
+  if (is_narrow(1, g)) { a.narrow_begin = 0; a.narrow_count = batch_size * nsplit; }
+  else { a.vnode_begin = 0; a.vnode_count = batch_size * nsplit; }
   a.g = g;
   a.hkv = num_kv_heads;
   a.scale_log2 = sm_scale * kLog2e;
   a.mid_o = mid_o; a.so0 = (int64_t)num_qo_heads * head_dim; a.so1 = head_dim;
   a.mid_lse = mid_lse; a.sl0 = num_qo_heads;
   a.cache_seqlens = cache_seqlens; a.max_seqlen = max_seqlen; a.kv_split = kv_split; a.nsplit = nsplit;
-  if (int rc = launch_stage1<true>(a, num_kv_heads, head_dim, g > 64 ? 64 : g, dtype, stream)) return rc;
+  if (int rc = launch_stage1<true>(a, head_dim, dtype, stream)) return rc;
   Stage2Args b{};
   b.mid_o = mid_o; b.so0 = a.so0; b.so1 = a.so1; b.mid_lse = mid_lse; b.sl0 = a.sl0;
   b.o = static_cast<char*>(o); b.oo0 = oo0; b.oo1 = oo1;

@@ -26,6 +26,8 @@ SIGNATURES = {
     "ft_error_string": (c_char_p, [c_int]),
     "ft_stage1": (c_int, [_P, _P, _P] + _I64x6 + [_P] * 6 + [c_int] * 7 + [c_float]
                   + [_P, c_int64, c_int64, _P, c_int64, c_int, _P]),
+    "ft_stage1_phases": (c_int, [_P, _P, _P] + _I64x6 + [_P] * 6 + [_P, c_int64, c_int64, _P, c_int64] + [_P] * 4
+                         + [c_int] * 3 + [c_float, c_int, _P]),
     "ft_stage2": (c_int, [_P, _P, _P, _P, c_int64, c_int64, _P, c_int64, _P, c_int64, c_int64,
                           c_int, c_int, c_int, c_int, _P]),
     "ft_decode": (c_int, [_P, _P, _P, _P] + [c_int64] * 8 + [_P] * 9

@@ -90,20 +90,37 @@ def fasttree_decode_stage1(q, k_buffer, v_buffer, vnode_to_kv_entries, vnode_to_
     (the role of _fasttree_decode_stage1, kernel_bench/fasttree.py:416-479)."""
     _need_gpu(q, k_buffer, v_buffer, mid_o, mid_lse)
     lib = _lib.load()
+    rc = lib.ft_stage1_phases(
+        q.data_ptr(), k_buffer.data_ptr(), v_buffer.data_ptr(),
+        q.stride(0), q.stride(1), k_buffer.stride(0), k_buffer.stride(1), v_buffer.stride(0), v_buffer.stride(1),
+        vnode_to_kv_entries.data_ptr(), vnode_to_kv_offs.data_ptr(), vnode_to_kv_lens.data_ptr(),
+        vnode_to_q_entries.data_ptr(), vnode_to_q_offs.data_ptr(), vnode_to_q_lens.data_ptr(),
+        mid_o.data_ptr(), mid_o.stride(0), mid_o.stride(1), mid_lse.data_ptr(), mid_lse.stride(0),
+        _lib.int32_pair(phase_node_nums), _lib.int32_pair(phase_node_offsets),
+        _lib.int32_pair(phase_q_tile_sizes), _lib.int32_pair(phase_kv_tile_sizes),
+        q.shape[1], k_buffer.shape[1], q.shape[-1], float(sm_scale), _dtype_code(q), _stream_handle(q),
+    )
+    _lib.check(rc, "ft_stage1_phases")
+
+
+def fasttree_decode_phase(q, k_buffer, v_buffer, vnode_to_kv_entries, vnode_to_kv_offs, vnode_to_kv_lens,
+                          vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, sm_scale, mid_o, mid_lse,
+                          node_num, node_offset, q_tile, kv_tile):
+    """One phase of stage 1 on its own: what one iteration of the reference's launch loop does
+    (kernel_bench/fasttree.py:443-479)."""
+    _need_gpu(q, k_buffer, v_buffer, mid_o, mid_lse)
+    lib = _lib.load()
     hq, hkv = q.shape[1], k_buffer.shape[1]
-    for num, off, qt, kt in zip(phase_node_nums, phase_node_offsets, phase_q_tile_sizes, phase_kv_tile_sizes):
-        if num == 0:
-            continue
-        rc = lib.ft_stage1(
-            q.data_ptr(), k_buffer.data_ptr(), v_buffer.data_ptr(),
-            q.stride(0), q.stride(1), k_buffer.stride(0), k_buffer.stride(1), v_buffer.stride(0), v_buffer.stride(1),
-            vnode_to_kv_entries.data_ptr(), vnode_to_kv_offs.data_ptr(), vnode_to_kv_lens.data_ptr(),
-            vnode_to_q_entries.data_ptr(), vnode_to_q_offs.data_ptr(), vnode_to_q_lens.data_ptr(),
-            int(off), int(num), hkv, hq // hkv, q.shape[-1], int(qt), int(kt), float(sm_scale),
-            mid_o.data_ptr(), mid_o.stride(0), mid_o.stride(1), mid_lse.data_ptr(), mid_lse.stride(0),
-            _dtype_code(q), _stream_handle(q),
-        )
-        _lib.check(rc, "ft_stage1")
+    rc = lib.ft_stage1(
+        q.data_ptr(), k_buffer.data_ptr(), v_buffer.data_ptr(),
+        q.stride(0), q.stride(1), k_buffer.stride(0), k_buffer.stride(1), v_buffer.stride(0), v_buffer.stride(1),
+        vnode_to_kv_entries.data_ptr(), vnode_to_kv_offs.data_ptr(), vnode_to_kv_lens.data_ptr(),
+        vnode_to_q_entries.data_ptr(), vnode_to_q_offs.data_ptr(), vnode_to_q_lens.data_ptr(),
+        int(node_offset), int(node_num), hkv, hq // hkv, q.shape[-1], int(q_tile), int(kv_tile), float(sm_scale),
+        mid_o.data_ptr(), mid_o.stride(0), mid_o.stride(1), mid_lse.data_ptr(), mid_lse.stride(0),
+        _dtype_code(q), _stream_handle(q),
+    )
+    _lib.check(rc, "ft_stage1")
 
 
 def fasttree_decode_stage2(req_to_vnode_entries, req_to_vnode_offs, req_to_vnode_lens, mid_o, mid_lse, o):

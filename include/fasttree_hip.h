@@ -70,6 +70,23 @@ int ft_stage1(const void* q, const void* k, const void* v,
               int dtype, ft_stream_t stream);
 
 /*
+ * Stage 1 for both phases in ONE launch: blocks for the wide phase first, then one wave per
+ * (vnode, KV head) of the narrow phase, so the short narrow items fill the machine while the
+ * wide blocks drain.  Replaces the whole of _fasttree_decode_stage1 (kernel_bench/fasttree.py:
+ * 416-479); phase_* are its four 2-element python lists.
+ */
+int ft_stage1_phases(const void* q, const void* k, const void* v,
+                     int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+                     const int32_t* vnode_to_kv_entries, const int32_t* vnode_to_kv_offs,
+                     const int32_t* vnode_to_kv_lens, const int32_t* vnode_to_q_entries,
+                     const int32_t* vnode_to_q_offs, const int32_t* vnode_to_q_lens,
+                     float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
+                     const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
+                     const int32_t phase_q_tile_sizes[2], const int32_t phase_kv_tile_sizes[2],
+                     int num_qo_heads, int num_kv_heads, int head_dim,
+                     float sm_scale, int dtype, ft_stream_t stream);
+
+/*
  * Stage 2: per (request, query head) log-sum-exp weighted merge of the request's
  * partial rows into o.  Replaces _fwd_fasttree_decoding_stage2 / _fasttree_decode_stage2
  * (kernel_bench/fasttree.py:482-579).
@@ -81,7 +98,7 @@ int ft_stage2(const int32_t* req_to_vnode_entries, const int32_t* req_to_vnode_o
               int batch_size, int num_qo_heads, int head_dim, int dtype, ft_stream_t stream);
 
 /*
- * The whole decode call: stage 1 for both phases, then stage 2.  Replaces
+ * The whole decode call: ft_stage1_phases, then ft_stage2.  Replaces
  * fasttree_decode (kernel_bench/fasttree.py:582-642); phase_* are its four 2-element
  * python lists.
  */
