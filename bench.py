@@ -116,6 +116,9 @@ def main():
     ap.add_argument("--no-gathered", action="store_true")
     ap.add_argument("--profile-only", action="store_true",
                     help="run warm-up + steps back to back and exit (for rocprofv3)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run a plain 256 MiB device copy a few times and exit: the known-size kernel the "
+                         "FETCH_SIZE / WRITE_SIZE counters are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build runs on ONE GPU; --gpus above 1 is not supported "
@@ -130,6 +133,14 @@ def main():
 
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.calibrate_copy:
+        src = torch.ones(1 << 26, dtype=torch.int32, device=device)   # 256 MiB
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        log("calibrate-copy: 5 copies of 268435456 bytes (read 256 MiB + write 256 MiB each)")
+        return
     if args.q_tiles or args.kv_splits:
         custom = dict(PRESETS[args.preset])
         if args.q_tiles:
