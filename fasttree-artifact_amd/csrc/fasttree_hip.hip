@@ -309,8 +309,11 @@ __device__ __forceinline__ void tile_step(const char* ldsK, const char* ldsV, in
 }
 
 // One wave attends NQB*16 query rows to tokens [tile0*32, ...) in steps of tile_step_n tiles,
-// staging each tile in its own LDS area.
-template <typename E, int D, int NQB, bool GATHERED>
+// staging each tile in its own LDS area.  Rows travel global -> registers -> LDS.  With DEEP,
+// the rows of the next two tiles and the slot indices of the two after those are in flight while
+// a tile is consumed, so a short run (the common leaf vnode) has all of its loads issued at
+// once instead of paying one memory round trip per tile; without it, one tile is in flight.
+template <typename E, int D, int NQB, bool GATHERED, bool DEEP = false>
 __device__ __forceinline__ void wave_attend(const Stage1Args& a, const VnodeView& vn, int kvh, int row0,
                                             int tile0, int tile_step_n, char* lds, WaveState<D, NQB>& st) {
   using G = TileGeom<D>;
@@ -325,27 +328,32 @@ __device__ __forceinline__ void wave_attend(const Stage1Args& a, const VnodeView
   const int ntiles = (vn.kv_len + kTileTokens - 1) / kTileTokens;
   if (tile0 >= ntiles) return;
 
-  // ---- global -> register prefetch of one tile (rows by 16-byte chunks, coalesced per row)
+  // rows by 16-byte chunks, coalesced per row
   const int ld_row = lane / G::kLanesPerRow, ld_chunk = lane % G::kLanesPerRow;
-  u32x4 kreg[G::kLoads], vreg[G::kLoads];
-  auto fetch = [&](int tile) {
+  const char* kbase = a.k + 2 * ((int64_t)kvh * a.sk1) + 16 * ld_chunk;
+  const char* vbase = a.v + 2 * ((int64_t)kvh * a.sv1) + 16 * ld_chunk;
+  auto load_slots = [&](int tile, int (&slot)[G::kLoads]) {
 #pragma unroll
     for (int i = 0; i < G::kLoads; ++i) {
       const int t = tile * kTileTokens + i * G::kRowsPerLoad + ld_row;
+      slot[i] = -1;
+      if (tile < ntiles && t < vn.kv_len) slot[i] = GATHERED ? t : a.kv_entries[vn.kv_base + t];
+    }
+  };
+  auto load_rows = [&](const int (&slot)[G::kLoads], u32x4 (&kreg)[G::kLoads], u32x4 (&vreg)[G::kLoads]) {
+#pragma unroll
+    for (int i = 0; i < G::kLoads; ++i) {
       u32x4 z = {0u, 0u, 0u, 0u};
       kreg[i] = z;
       vreg[i] = z;
-      if (t < vn.kv_len) {
-        const int64_t slot = GATHERED ? (vn.kv_base + t) : (int64_t)a.kv_entries[vn.kv_base + t];
-        kreg[i] = *reinterpret_cast<const u32x4*>(a.k + 2 * (slot * a.sk0 + (int64_t)kvh * a.sk1) + 16 * ld_chunk);
-        vreg[i] = *reinterpret_cast<const u32x4*>(a.v + 2 * (slot * a.sv0 + (int64_t)kvh * a.sv1) + 16 * ld_chunk);
+      if (slot[i] >= 0) {
+        const int64_t srow = GATHERED ? (vn.kv_base + slot[i]) : (int64_t)slot[i];
+        kreg[i] = *reinterpret_cast<const u32x4*>(kbase + 2 * srow * a.sk0);
+        vreg[i] = *reinterpret_cast<const u32x4*>(vbase + 2 * srow * a.sv0);
       }
     }
   };
-  fetch(tile0);
-
-  for (int tile = tile0; tile < ntiles; tile += tile_step_n) {
-    // registers -> this wave's LDS tile
+  auto stage = [&](const u32x4 (&kreg)[G::kLoads], const u32x4 (&vreg)[G::kLoads]) {
 #pragma unroll
     for (int i = 0; i < G::kLoads; ++i) {
       const int row = i * G::kRowsPerLoad + ld_row;
@@ -353,9 +361,46 @@ __device__ __forceinline__ void wave_attend(const Stage1Args& a, const VnodeView
       *reinterpret_cast<u32x4*>(ldsV + row * G::kPitchV + 16 * ld_chunk) = vreg[i];
     }
     wave_lds_fence();
-    if (tile + tile_step_n < ntiles) fetch(tile + tile_step_n);
-    tile_step<E, D, NQB>(ldsK, ldsV, vn.kv_len - tile * kTileTokens, a.scale_log2, qf, st);
-    wave_lds_fence();
+  };
+
+  if constexpr (!DEEP) {
+    int slot[G::kLoads];
+    u32x4 kreg[G::kLoads], vreg[G::kLoads];
+    load_slots(tile0, slot);
+    load_rows(slot, kreg, vreg);
+    for (int tile = tile0; tile < ntiles; tile += tile_step_n) {
+      stage(kreg, vreg);
+      if (tile + tile_step_n < ntiles) {
+        load_slots(tile + tile_step_n, slot);
+        load_rows(slot, kreg, vreg);
+      }
+      tile_step<E, D, NQB>(ldsK, ldsV, vn.kv_len - tile * kTileTokens, a.scale_log2, qf, st);
+      wave_lds_fence();
+    }
+  } else {
+    // even tiles use set 0, odd tiles set 1 (tile numbering relative to tile0, step tile_step_n)
+    int slot0[G::kLoads], slot1[G::kLoads];
+    u32x4 k0[G::kLoads], v0[G::kLoads], k1[G::kLoads], v1[G::kLoads];
+    const int dt = tile_step_n;
+    load_slots(tile0, slot0);
+    load_slots(tile0 + dt, slot1);
+    load_rows(slot0, k0, v0);
+    load_rows(slot1, k1, v1);
+    load_slots(tile0 + 2 * dt, slot0);
+    load_slots(tile0 + 3 * dt, slot1);
+    for (int tile = tile0; tile < ntiles; tile += 2 * dt) {
+      stage(k0, v0);
+      load_rows(slot0, k0, v0);                 // tile + 2*dt
+      load_slots(tile + 4 * dt, slot0);
+      tile_step<E, D, NQB>(ldsK, ldsV, vn.kv_len - tile * kTileTokens, a.scale_log2, qf, st);
+      wave_lds_fence();
+      if (tile + dt >= ntiles) break;
+      stage(k1, v1);
+      load_rows(slot1, k1, v1);                 // tile + 3*dt
+      load_slots(tile + 5 * dt, slot1);
+      tile_step<E, D, NQB>(ldsK, ldsV, vn.kv_len - (tile + dt) * kTileTokens, a.scale_log2, qf, st);
+      wave_lds_fence();
+    }
   }
   finish_state<D, NQB>(st);
 }
@@ -846,13 +891,19 @@ __global__ void __launch_bounds__(kWideBlock) stage1_fused_kernel(Stage1Args a) 
     if (item >= a.narrow_count * a.hkv) return;  // whole wave; no block barrier below
     const int local_vnode = item / a.hkv;
     const int kvh = item - local_vnode * a.hkv;
+    FT_TIME(unsigned long long t_start = FT_CLOCK(); unsigned long long rt_start = wall_clock64();)
     const VnodeView vn = load_vnode<GATHERED>(a, a.narrow_begin + local_vnode);
     const int rows_total = vn.q_len * a.g;
     for (int row0 = 0; row0 < rows_total; row0 += 16) {
       WaveState<D, 1> st;
-      wave_attend<E, D, 1, GATHERED>(a, vn, kvh, row0, 0, 1, smem + wave * TileGeom<D>::kBytes, st);
+      // (the gathered baseline streams long contiguous runs: one tile in flight is enough there)
+      wave_attend<E, D, 1, GATHERED, !GATHERED>(a, vn, kvh, row0, 0, 1, smem + wave * TileGeom<D>::kBytes, st);
       write_partials<D, 1>(a, vn, kvh, row0, st);
     }
+    FT_TIME(if (g_timing && (threadIdx.x & 63) == 0) {
+      unsigned long long* out = g_timing + ((size_t)blockIdx.x * kWideWaves + wave) * 8;
+      out[4] = FT_CLOCK() - t_start; out[5] = 0; out[6] = rt_start; out[7] = wall_clock64();
+    })
   }
 }
 
