@@ -514,6 +514,7 @@ __global__ void __launch_bounds__(kBlock) stage1_kernel(Stage1Args a) {
 // Development aid, compiled out of the product: per-wave cycle counts of the wide kernel's
 // phases, written to a buffer set with ft_debug_set_timing().
 __device__ unsigned long long* g_timing = nullptr;
+__device__ int g_timing_steps = 0;  // 1: report per-step phases (scores, soft-max, P.V, steps) instead
 #define FT_CLOCK() __builtin_readcyclecounter()
 #define FT_TIME(...) __VA_ARGS__
 #else
@@ -522,23 +523,29 @@ __device__ unsigned long long* g_timing = nullptr;
 constexpr int kWideWaves = 8;
 constexpr int kWideBlock = kWave * kWideWaves;
 
-// LDS layout of the wide kernel: rows of 2*D bytes back to back (no padding), 128-token super
-// tiles of four 32-token tiles, two buffers.  A row's 16-byte chunks are stored XOR-permuted:
-// chunk c of row r sits in slot c ^ swz(r).  swz swaps the two low bit pairs of r, which makes
-// both read patterns conflict free for 256-byte rows: the K operand read (16 different rows,
-// same chunk) and the transposed V read (4 consecutive rows x 4 consecutive chunks).
-// Loads go global -> LDS directly; one wave instruction fills a 1 KB group of consecutive rows.
+// LDS layout of the wide kernel: rows of 2*D bytes back to back (no padding), 64-token super
+// tiles of two 32-token tiles, a ring of four buffers, then a staging area for the run's slot
+// indices.  A row's 16-byte chunks are stored XOR-permuted: chunk c of row r sits in slot
+// c ^ swz(r).  swz swaps the two low bit pairs of r, which makes both read patterns conflict free
+// for 256-byte rows: the K operand read (16 different rows, same chunk) and the transposed V
+// read (4 consecutive rows x 4 consecutive chunks).  Loads go global -> LDS directly; one wave
+// instruction fills a 1 KB group of consecutive rows.
 template <int D> struct WideGeom {
   static constexpr int kRowBytes = 2 * D;
   static constexpr int kChunks = D / 8;                  // 16-byte chunks per row
-  static constexpr int kSub = 4;
-  static constexpr int kTokens = kSub * kTileTokens;     // 128
+  static constexpr int kSub = 2;
+  static constexpr int kTokens = kSub * kTileTokens;     // 64
+  static constexpr int kBufs = 4;
   static constexpr int kTileBytes = kTileTokens * kRowBytes;
   static constexpr int kBytesK = kTokens * kRowBytes;
-  static constexpr int kBytes = 2 * kBytesK;             // K + V of one buffer (a power of two)
+  static constexpr int kBytes = 2 * kBytesK;             // K + V of one buffer
+  static constexpr int kRing = kBufs * kBytes;           // a power of two
   static constexpr int kGroupRows = kWave / kChunks;     // rows per 1 KB load group
-  static constexpr int kGroups = kTokens / kGroupRows;
-  static constexpr int kGroupsPerWave = kGroups / kWideWaves;
+  static constexpr int kGroups = kTokens / kGroupRows;   // groups per matrix and super tile
+  static constexpr int kUnits = 2 * kGroups / kWideWaves;                       // loads per wave and super tile
+  static constexpr int kSlots = kGroups >= kWideWaves ? kGroups / kWideWaves : 1;  // distinct rows among them
+  static constexpr int kIdxCap = 4096;                   // slot indices staged at a time (tokens)
+  static constexpr int kLds = kRing + 4 * kIdxCap;
   static __device__ __forceinline__ int swz(int row) { return (((row & 3) << 2) | ((row >> 2) & 3)) & (kChunks - 1); }
 };
 
@@ -579,11 +586,11 @@ __device__ __forceinline__ void load_q_frags32(const Stage1Args& a, const VnodeV
   }
 }
 
-// Per-lane LDS byte addresses of the operand reads inside tile 0 of buffer 0, for contraction
-// step / dim block 0.  Thanks to the XOR layout the address for step ks (dim block db) is the
-// base with 32*ks (64*db) XOR-ed in; other tiles of the super tile are a constant offset away
-// and the other buffer is reached by flipping bit log2(kBytes) (the buffers are kBytes apart,
-// kBytes is a power of two and the dynamic LDS segment starts at 0).
+// Per-lane LDS byte addresses of the operand reads inside tile 0 of the current buffer, for
+// contraction step / dim block 0.  Thanks to the XOR layout the address for step ks (dim block
+// db) is the base with 32*ks (64*db) XOR-ed in; the second tile of the super tile is a constant
+// offset away and the next buffer of the ring is kBytes further, modulo the ring size (the
+// dynamic LDS segment starts at 0).
 struct WideLane {
   unsigned k;     // K operand: row lane%32, chunk lane/32 (step ks: chunk 2*ks + lane/32)
   unsigned v_lo;  // transposed V read: tokens 4*(lane/32) + 0..3 (+16 for u = 1), dims 0..31
@@ -603,11 +610,26 @@ __device__ __forceinline__ void init_lane(WideLane& la) {
 }
 
 template <int D>
-__device__ __forceinline__ void flip_buffer(WideLane& la) {
+__device__ __forceinline__ void next_buffer(WideLane& la) {
   using W = WideGeom<D>;
-  la.k ^= W::kBytes;
-  la.v_lo ^= W::kBytes;
-  la.v_hi ^= W::kBytes;
+  la.k = (la.k + W::kBytes) & (W::kRing - 1);
+  la.v_lo = (la.v_lo + W::kBytes) & (W::kRing - 1);
+  la.v_hi = (la.v_hi + W::kBytes) & (W::kRing - 1);
+}
+
+// 16 bytes per lane from global memory straight into LDS at lds_base + 16 * lane (lds_base is
+// wave uniform).  Written as assembly on purpose: for the builtin the compiler cannot tell which
+// later LDS reads touch the landing bytes and makes every one of them wait for all such loads
+// in flight, which serialises the stream with the arithmetic.  Completion is awaited by hand
+// with wait_direct_loads<N>() before the block barrier that publishes a buffer.
+__device__ __forceinline__ void load_direct16(const char* src, unsigned lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_base) : "memory");
+}
+// Wait until at most N of this wave's vector-memory operations are still in flight (they finish
+// in order).
+template <int N>
+__device__ __forceinline__ void wait_direct_loads() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
 __device__ __forceinline__ u32x4 lds_read16(unsigned addr) {
@@ -629,11 +651,12 @@ constexpr float kSlack = 8.f;
 // S^T = K Q^T: A = K rows (token lane%32, 8 dims per lane), B = Q; accumulator register j of a
 // lane is token 8*(j/4) + 4*(lane/32) + j%4.  Registers 8u .. 8u+7 are exactly the 8 k-slots a
 // lane feeds to the u-th P.V contraction, whose A operand (V^T) comes from two transposed LDS
-// reads of 4 consecutive tokens each.  MASKED is used for a run's last, partial tile only.
-template <typename E, int D, bool MASKED>
+// reads of 4 consecutive tokens each.  valid < 32 only on a run's last, partial tile.
+template <typename E, int D>
 __device__ __forceinline__ void tile_step32(const WideLane& la, unsigned off, int valid, float sc,
-                                            const u32x4 (&qf)[D / 16], WideState<D>& st) {
+                                            const u32x4 (&qf)[D / 16], WideState<D>& st FT_TIME(, unsigned long long* tt = nullptr)) {
   using W = WideGeom<D>;
+  FT_TIME(const unsigned long long tc0 = FT_CLOCK();)
   constexpr int KS = D / 16, DB = D / 32, NV = 2 * DB;
 
   // all K operands of the tile are requested before the first contraction needs one
@@ -650,12 +673,14 @@ __device__ __forceinline__ void tile_step32(const WideLane& la, unsigned off, in
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) s = E::mfma32(kf[ks], qf[ks], s);
 
-  if constexpr (MASKED) {
+  if (valid < kTileTokens) {  // wave uniform
+    asm volatile("" ::: "memory");  // keeps this a branch: as selects it would run on every tile
     const int h = (threadIdx.x & 63) >> 5;
 #pragma unroll
     for (int j = 0; j < 16; ++j) s[j] = (8 * (j >> 2) + 4 * h + (j & 3) >= valid) ? -INFINITY : s[j];
   }
 
+  FT_TIME(__builtin_amdgcn_sched_barrier(0); const unsigned long long tc1 = FT_CLOCK(); __builtin_amdgcn_sched_barrier(0);)
   float mx = max3(s[0], s[1], s[2]);
 #pragma unroll
   for (int j = 3; j < 15; j += 2) mx = max3(mx, s[j], s[j + 1]);
@@ -685,6 +710,7 @@ __device__ __forceinline__ void tile_step32(const WideLane& la, unsigned off, in
     pf[u] = u32x4{E::pack2(x[8 * u + 0], x[8 * u + 1]), E::pack2(x[8 * u + 2], x[8 * u + 3]),
                   E::pack2(x[8 * u + 4], x[8 * u + 5]), E::pack2(x[8 * u + 6], x[8 * u + 7])};
 
+  FT_TIME(__builtin_amdgcn_sched_barrier(0); const unsigned long long tc2 = FT_CLOCK(); __builtin_amdgcn_sched_barrier(0);)
   const unsigned vlo = la.v_lo + off, vhi = la.v_hi + off;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
@@ -694,6 +720,7 @@ __device__ __forceinline__ void tile_step32(const WideLane& la, unsigned off, in
     const u32x4 vf = {lo[0], lo[1], hi[0], hi[1]};
     st.o[db] = E::mfma32(vf, pf[u], st.o[db]);
   }
+  FT_TIME(if (tt) { __builtin_amdgcn_sched_barrier(0); const unsigned long long tc3 = FT_CLOCK(); tt[0] += tc1 - tc0; tt[1] += tc2 - tc1; tt[2] += tc3 - tc2; tt[3] += 1; })
 }
 
 template <int D>
@@ -759,16 +786,17 @@ __device__ __forceinline__ void merge_token_groups(float* xchg, WideState<D>& st
   }
 }
 
-// One block (8 waves) per (vnode, kv head).  The block streams the vnode's KV run through LDS
-// 128 tokens at a time with direct global->LDS loads; the next super tile is in flight while
-// the current one is consumed.  Per pass over the run the waves form RG row groups of 32 query
-// rows x TG token groups (RG * TG = 8, or 4 when only 32 rows are left): a wave consumes the
-// tiles tg, tg + TG, .. of every super tile for the rows of its row group, and the TG states of
-// a row group are merged at the end.
+// One block (8 waves) per (vnode, kv head).  The block streams the vnode's KV run through a ring
+// of four 64-token LDS buffers with direct global->LDS loads, three super tiles ahead of the one
+// being consumed; the run's slot indices are staged in LDS first so that nothing but those
+// loads is in flight in the loop.  Per pass over the run the waves form RG row groups of 32
+// query rows x TG token groups (RG * TG = 8, or 4 when only 32 rows are left): a wave consumes
+// the 32-token tiles t with t % TG == tg for the rows of its row group, and the TG states of a
+// row group are merged at the end.
 template <typename E, int D, bool GATHERED>
 __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int local_vnode, int kvh) {
   using W = WideGeom<D>;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const VnodeView vn = load_vnode<GATHERED>(a, a.vnode_begin + local_vnode);
   const int rows_total = vn.q_len * a.g;
   const int nsuper = (vn.kv_len + W::kTokens - 1) / W::kTokens;
@@ -777,6 +805,8 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
   const int grp_row = lane / W::kChunks, pos = lane % W::kChunks;
   const char* kbase = a.k + 2 * ((int64_t)kvh * a.sk1);
   const char* vbase = a.v + 2 * ((int64_t)kvh * a.sv1);
+  const unsigned k_stride = (unsigned)(2 * a.sk0), v_stride = (unsigned)(2 * a.sv0);  // bytes, < 2^32 (checked by the host)
+  int* idx_lds = reinterpret_cast<int*>(smem + W::kRing);
 
   for (int row0 = 0; row0 < rows_total;) {
     const int groups = (rows_total - row0 + 31) >> 5;   // 32-row groups still to serve
@@ -793,74 +823,87 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
     WideLane la;
     init_lane<D>(la);
 
-    // slots of the rows this lane loads in the next super tile (group g = j*8 + wave)
-    int slot[W::kGroupsPerWave];
-    auto load_slots = [&](int super) {
+    // slot indices of tokens [idx_base, idx_base + kIdxCap) of the run, staged by the whole block
+    int idx_base = 0;
+    auto stage_indices = [&](int base) {
+      if constexpr (!GATHERED) {
+        idx_base = base;
+        // (branch free, so that the loads are in flight together; entries past the run repeat its last)
+        int e[W::kIdxCap / kWideBlock];
 #pragma unroll
-      for (int j = 0; j < W::kGroupsPerWave; ++j) {
-        const int t = super * W::kTokens + (j * kWideWaves + wave) * W::kGroupRows + grp_row;
-        slot[j] = -1;
-        if (t < vn.kv_len) slot[j] = GATHERED ? (int)t : a.kv_entries[vn.kv_base + t];
+        for (int i = 0; i < W::kIdxCap / kWideBlock; ++i)
+          e[i] = a.kv_entries[vn.kv_base + min(base + kWideBlock * i + (int)threadIdx.x, vn.kv_len - 1)];
+#pragma unroll
+        for (int i = 0; i < W::kIdxCap / kWideBlock; ++i) idx_lds[kWideBlock * i + threadIdx.x] = e[i];
+        __syncthreads();
       }
     };
-    auto issue_rows = [&](int super) {
-      char* bufK = smem + (super & 1) * W::kBytes;
-      char* bufV = bufK + W::kBytesK;
-#pragma unroll
-      for (int j = 0; j < W::kGroupsPerWave; ++j) {
-        const int grp = j * kWideWaves + wave;
-        const int row = grp * W::kGroupRows + grp_row;
-        const int chunk = pos ^ W::swz(row);
-        char* dstK = bufK + grp * 1024;   // wave-uniform; lane l lands at +16*l
-        char* dstV = bufV + grp * 1024;
-        if (slot[j] >= 0) {
-          const int64_t srow = GATHERED ? (vn.kv_base + slot[j]) : (int64_t)slot[j];
-          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kbase + 2 * srow * a.sk0 + 16 * chunk),
-                                           (__attribute__((address_space(3))) void*)dstK, 16, 0, 0);
-          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vbase + 2 * srow * a.sv0 + 16 * chunk),
-                                           (__attribute__((address_space(3))) void*)dstV, 16, 0, 0);
-        } else {
-          // rows past the run: V must be finite (it meets zero probabilities), K is masked later
-          *reinterpret_cast<u32x4*>(dstV + 16 * lane) = u32x4{0u, 0u, 0u, 0u};
+    // rows of super tile j -> ring buffer j % 4.  Tokens past the run repeat its last token: the
+    // scores of such rows are masked and their V rows are finite.
+    auto issue_rows = [&](int j) {
+      if (j >= nsuper) return;
+      if constexpr (!GATHERED) {
+        if (j * W::kTokens >= idx_base + W::kIdxCap) {  // block uniform
+          __syncthreads();                              // every wave has read the indices it needed
+          stage_indices(idx_base + W::kIdxCap);
         }
       }
+      const unsigned buf = (unsigned)(j & (W::kBufs - 1)) * W::kBytes;
+      unsigned srow[W::kSlots];
+      unsigned chunk[W::kSlots];
+#pragma unroll
+      for (int u = 0; u < W::kSlots; ++u) {
+        const int grp = W::kGroups >= kWideWaves ? u * kWideWaves + wave : wave % W::kGroups;
+        const int row = grp * W::kGroupRows + grp_row;
+        const int t = min(j * W::kTokens + row, vn.kv_len - 1);
+        srow[u] = GATHERED ? (unsigned)(vn.kv_base + t) : (unsigned)idx_lds[t - idx_base];
+        chunk[u] = 16 * (pos ^ W::swz(row));
+      }
+#pragma unroll
+      for (int u = 0; u < W::kUnits; ++u) {
+        // unit u of this wave: K groups first, then V groups
+        const bool is_v = W::kGroups >= kWideWaves ? u >= W::kSlots : wave >= W::kGroups;
+        const int sl = u % W::kSlots;
+        const int grp = W::kGroups >= kWideWaves ? sl * kWideWaves + wave : wave % W::kGroups;
+        const char* src = (is_v ? vbase : kbase) + (uint64_t)srow[sl] * (is_v ? v_stride : k_stride);
+        load_direct16(src + chunk[sl], buf + (is_v ? W::kBytesK : 0) + grp * 1024);
+      }
     };
-    if (nsuper > 0) {
-      load_slots(0);
-      issue_rows(0);
-      if (nsuper > 1) load_slots(1);
-    }
-    FT_TIME(unsigned long long t_start = FT_CLOCK(); unsigned long long rt_start = wall_clock64(); unsigned long long t_wait = 0, t_bar = 0, t_issue = 0, t_comp = 0;)
+    if (nsuper > 0) stage_indices(0);  // block uniform
+    // nothing the compiler itself tracks (the Q fragments) may still be in flight in the loop:
+    // a wait for it there would also wait for every direct load
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    issue_rows(0);
+    issue_rows(1);
+    issue_rows(2);
+    FT_TIME(unsigned long long t_start = FT_CLOCK(); unsigned long long rt_start = wall_clock64(); unsigned long long t_wait = 0, t_bar = 0, t_issue = 0, t_comp = 0; unsigned long long t_step[4] = {0, 0, 0, 0};)
     for (int super = 0; super < nsuper; ++super) {
-      // the loads of this super tile were issued one iteration ago; publish them to the block
+      // publish super tile `super` to the block; the two after it may stay in flight
       FT_TIME(unsigned long long c0 = FT_CLOCK();)
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      if (super + 2 < nsuper) wait_direct_loads<2 * W::kUnits>();
+      else if (super + 1 < nsuper) wait_direct_loads<W::kUnits>();
+      else wait_direct_loads<0>();
       FT_TIME(unsigned long long c1 = FT_CLOCK();)
       __syncthreads();
       FT_TIME(unsigned long long c2 = FT_CLOCK();)
-      // the other buffer was last read before that barrier: refill it now
-      if (super + 1 < nsuper) {
-        issue_rows(super + 1);
-        if (super + 2 < nsuper) load_slots(super + 2);
-      }
+      // the buffer consumed before that barrier is free: refill it
+      issue_rows(super + 3);
       FT_TIME(unsigned long long c3 = FT_CLOCK();)
       if (active) {
-        const int left = vn.kv_len - super * W::kTokens;  // tokens from the start of this super tile
 #pragma unroll 1
-        for (int sub = tg; sub < W::kSub; sub += tgroups) {
-          const int valid = left - sub * kTileTokens;
-          if (valid >= kTileTokens)
-            tile_step32<E, D, false>(la, sub * W::kTileBytes, valid, a.scale_log2, qf, st);
-          else if (valid > 0)
-            tile_step32<E, D, true>(la, sub * W::kTileBytes, valid, a.scale_log2, qf, st);
+        for (int sub = 0; sub < W::kSub; ++sub) {
+          const int tile = super * W::kSub + sub;
+          if ((tile & (tgroups - 1)) != tg) continue;
+          const int valid = vn.kv_len - tile * kTileTokens;
+          if (valid > 0) tile_step32<E, D>(la, sub * W::kTileBytes, valid, a.scale_log2, qf, st FT_TIME(, t_step));
         }
       }
-      flip_buffer<D>(la);
+      next_buffer<D>(la);
       FT_TIME(unsigned long long c4 = FT_CLOCK(); t_wait += c1 - c0; t_bar += c2 - c1; t_issue += c3 - c2; t_comp += c4 - c3;)
     }
     FT_TIME(if (g_timing && lane == 0) {
       unsigned long long* out = g_timing + ((size_t)(local_vnode * a.hkv + kvh) * kWideWaves + wave) * 8;
-      out[0] = t_wait; out[1] = t_bar; out[2] = t_issue; out[3] = t_comp; out[4] = FT_CLOCK() - t_start; out[5] = nsuper;
+      out[0] = g_timing_steps ? t_step[0] : t_wait; out[1] = g_timing_steps ? t_step[1] : t_bar; out[2] = g_timing_steps ? t_step[2] : t_issue; out[3] = g_timing_steps ? t_step[3] : t_comp; out[4] = FT_CLOCK() - t_start; out[5] = nsuper;
       out[6] = rt_start; out[7] = wall_clock64();
     })
     finish_state<D>(st);
@@ -871,35 +914,224 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
   }
 }
 
-// Stage 1 in one launch.  Blocks [0, wide vnodes x KV heads) serve the wide vnodes, one block
-// per (vnode, KV head); the blocks after them serve the narrow vnodes, one wave per (vnode, KV
-// head).  The KV head varies fastest: blocks are handed to the 8 XCDs round robin, so with 8 KV
-// heads every head's KV stays in one XCD's L2.  The wide vnodes start first, in list order (the
-// planner lists the widest, longest ones first); the many short narrow items then fill the
-// compute units as the wide blocks drain, and their HBM-bound streaming overlaps the
-// matrix-bound tail.
+// ---------------------------------------------------------------------------------------
+// Narrow vnodes (at most 16 query rows): one wave per (vnode, kv head) streams the run through
+// a wave-private LDS tile of 32 tokens with direct global->LDS loads, in the same unpadded XOR
+// layout as the wide kernel.  K and V have one tile each: the K rows of the next tile are
+// requested as soon as the scores of the current one are out of LDS, its V rows as soon as the
+// current P.V is, so a leaf vnode of a few dozen tokens costs little more than its two memory
+// round trips (slot indices, rows).  Slot indices are staged 256 tokens at a time.
+// ---------------------------------------------------------------------------------------
+template <int D> struct NarrowGeom {
+  static constexpr int kRowBytes = 2 * D;
+  static constexpr int kChunks = D / 8;
+  static constexpr int kBytesK = kTileTokens * kRowBytes;
+  static constexpr int kBytes = 2 * kBytesK;
+  static constexpr int kGroupRows = kWave / kChunks;            // rows per 1 KB load
+  static constexpr int kGroups = kTileTokens / kGroupRows;      // loads per matrix and tile
+  static constexpr int kIdxCap = 256;
+  static constexpr int kLds = kBytes + 4 * kIdxCap;             // per wave; a multiple of the row size
+  static __device__ __forceinline__ int swz(int row) { return (((row & 3) << 2) | ((row >> 2) & 3)) & (kChunks - 1); }
+};
+
+template <typename E, int D, bool GATHERED>
+__device__ __forceinline__ void narrow_wave(const Stage1Args& a, char* smem, int wave, int vnode, int kvh) {
+  using N = NarrowGeom<D>;
+  constexpr int KS = D / 32, DB = D / 16;
+  constexpr float kSlackN = 8.f;
+  const int lane = threadIdx.x & 63;
+  const int p = lane & 15, c = lane >> 4;
+  const unsigned lds0 = (unsigned)wave * N::kLds;  // the dynamic LDS segment starts at 0
+  const VnodeView vn = load_vnode<GATHERED>(a, vnode);
+  const int rows_total = vn.q_len * a.g;
+  const int ntiles = (vn.kv_len + kTileTokens - 1) / kTileTokens;
+  int* idx_lds = reinterpret_cast<int*>(smem + lds0 + N::kBytes);
+
+  // loader role: 16-byte slot `pos` of row `grp_row` in each 1 KB group
+  const int grp_row = lane / N::kChunks, pos = lane % N::kChunks;
+  const char* kbase = a.k + 2 * ((int64_t)kvh * a.sk1);
+  const char* vbase = a.v + 2 * ((int64_t)kvh * a.sv1);
+  const unsigned k_stride = (unsigned)(2 * a.sk0), v_stride = (unsigned)(2 * a.sv0);  // bytes, < 2^32 (checked by the host)
+  unsigned src_off[N::kGroups];
+#pragma unroll
+  for (int g = 0; g < N::kGroups; ++g) src_off[g] = 16 * (pos ^ N::swz(g * N::kGroupRows + grp_row));
+
+  // operand read addresses: K row 16*tb + p, chunk c (contraction step ks: chunk 4*ks + c);
+  // V tokens 4*c + p/4 (+16), chunk 2*db + (p%4)/2, half p%2
+  unsigned k_addr[2], v_addr[2];
+#pragma unroll
+  for (int tb = 0; tb < 2; ++tb) {
+    const int kr = 16 * tb + p, vr = 16 * tb + 4 * c + (p >> 2);
+    k_addr[tb] = lds0 + kr * N::kRowBytes + 16 * ((c & (N::kChunks - 1)) ^ N::swz(kr));
+    v_addr[tb] = lds0 + N::kBytesK + vr * N::kRowBytes + 16 * ((((p & 3) >> 1) & (N::kChunks - 1)) ^ N::swz(vr)) + 8 * (p & 1);
+  }
+
+  for (int row0 = 0; row0 < rows_total; row0 += 16) {
+    u32x4 qf[1][KS];
+    load_q_frags<D, 1, GATHERED>(a, vn, kvh, row0, qf);
+    WaveState<D, 1> st;
+    reset_state<D, 1>(st);
+    if (ntiles > 0) {
+      int idx_base = 0;
+      auto stage_indices = [&](int base) {
+        if constexpr (!GATHERED) {
+          idx_base = base;
+          // (branch free, so that the loads are in flight together; entries past the run repeat its last)
+          int e[N::kIdxCap / kWave];
+#pragma unroll
+          for (int i = 0; i < N::kIdxCap / kWave; ++i)
+            e[i] = a.kv_entries[vn.kv_base + min(base + kWave * i + lane, vn.kv_len - 1)];
+#pragma unroll
+          for (int i = 0; i < N::kIdxCap / kWave; ++i) idx_lds[kWave * i + lane] = e[i];
+          wave_lds_fence();
+        }
+      };
+      // pool rows of the tokens this lane loads in `tile`; tokens past the run repeat its last
+      // token (their scores are masked, their V rows are finite)
+      unsigned srow[N::kGroups];
+      auto find_rows = [&](int tile) {
+        if constexpr (!GATHERED) {
+          if (tile * kTileTokens >= idx_base + N::kIdxCap) stage_indices(idx_base + N::kIdxCap);
+        }
+#pragma unroll
+        for (int g = 0; g < N::kGroups; ++g) {
+          const int t = min(tile * kTileTokens + g * N::kGroupRows + grp_row, vn.kv_len - 1);
+          srow[g] = GATHERED ? (unsigned)(vn.kv_base + t) : (unsigned)idx_lds[t - idx_base];
+        }
+      };
+      auto issue = [&](bool is_v) {
+#pragma unroll
+        for (int g = 0; g < N::kGroups; ++g) {
+          const char* src = (is_v ? vbase : kbase) + (uint64_t)srow[g] * (is_v ? v_stride : k_stride) + src_off[g];
+          load_direct16(src, lds0 + (is_v ? N::kBytesK : 0) + g * 1024);
+        }
+      };
+      stage_indices(0);
+      // nothing the compiler itself tracks may still be in flight below: a wait for it would
+      // also wait for every direct load
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      find_rows(0);
+      issue(false);
+      issue(true);
+      for (int tile = 0; tile < ntiles; ++tile) {
+        const bool more = tile + 1 < ntiles;
+        const int valid = vn.kv_len - tile * kTileTokens;
+        // ---- S^T = K Q^T : s[tb][j] = score(token 16*tb + 4*c + j, row p)
+        wait_direct_loads<N::kGroups>();  // K landed; V may still be in flight
+        f32x4 s[2];
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb) {
+          s[tb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) s[tb] = E::mfma(lds_read16(k_addr[tb] ^ (64u * ks)), qf[0][ks], s[tb]);
+        }
+        if (more) {
+          find_rows(tile + 1);
+          __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the K tile has been read
+          issue(false);
+        }
+        if (valid < kTileTokens) {
+#pragma unroll
+          for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              if (16 * tb + 4 * c + j >= valid) s[tb][j] = -INFINITY;
+        }
+        // online soft-max with a lazily updated reference (see tile_step)
+        float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
+                         fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+        mx = xor32_max(xor16_max(mx)) * a.scale_log2;
+        const bool grow = mx > st.m[0] + kSlackN;
+        if (__builtin_amdgcn_ballot_w64(grow)) {
+          const float m_new = grow ? mx : st.m[0];
+          const float alpha = __builtin_amdgcn_exp2f(st.m[0] - m_new);
+          st.l[0] *= alpha;
+#pragma unroll
+          for (int db = 0; db < DB; ++db) st.o[0][db] *= alpha;
+          st.m[0] = m_new;
+        }
+        const float neg_m = -st.m[0];
+        float x[8];
+        float sum = 0.f;
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            x[4 * tb + j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tb][j], a.scale_log2, neg_m));
+            sum += x[4 * tb + j];
+          }
+        st.l[0] += sum;
+        const u32x4 pf = {E::pack2(x[0], x[1]), E::pack2(x[2], x[3]), E::pack2(x[4], x[5]), E::pack2(x[6], x[7])};
+        // ---- O^T += V^T P^T
+        if (more) wait_direct_loads<N::kGroups>();  // V landed; the next K may be in flight
+        else wait_direct_loads<0>();
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const u32x2 lo = lds_read_tr8(v_addr[0] ^ (32u * db));
+          const u32x2 hi = lds_read_tr8(v_addr[1] ^ (32u * db));
+          const u32x4 vf = {lo[0], lo[1], hi[0], hi[1]};
+          st.o[0][db] = E::mfma(vf, pf, st.o[0][db]);
+        }
+        if (more) {
+          __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the V tile has been read
+          issue(true);
+        }
+      }
+    }
+    finish_state<D, 1>(st);
+    write_partials<D, 1>(a, vn, kvh, row0, st);
+  }
+}
+
+// Blocks are handed to compute units in index order as units become free, so serving the wide
+// vnodes in order of decreasing work (query rows x tokens) is longest-job-first list scheduling:
+// the machine does not end on a late start of a long block.  Every block ranks the wide vnodes
+// itself (they are few) and takes the one whose rank is `target`.  Block uniform.
+constexpr int kMaxRanked = kWideBlock;
+template <bool GATHERED>
+__device__ __forceinline__ int wide_vnode_of_rank(const Stage1Args& a, char* smem, int target) {
+  const int n = a.vnode_count;
+  if (n < 2 || n > kMaxRanked) return target;
+  unsigned long long* cost = reinterpret_cast<unsigned long long*>(smem);
+  int* found = reinterpret_cast<int*>(cost + kMaxRanked);
+  const int tid = threadIdx.x;
+  unsigned long long mine = 0;
+  if (tid < n) {
+    const VnodeView vn = load_vnode<GATHERED>(a, a.vnode_begin + tid);
+    mine = (unsigned long long)(unsigned)(vn.q_len * a.g) * (unsigned)vn.kv_len;
+    cost[tid] = mine;
+  }
+  __syncthreads();
+  if (tid < n) {
+    int rank = 0;
+    for (int j = 0; j < n; ++j) {
+      const unsigned long long c = cost[j];
+      rank += (c > mine || (c == mine && j < tid)) ? 1 : 0;
+    }
+    if (rank == target) *found = tid;
+  }
+  __syncthreads();
+  const int v = *found;
+  __syncthreads();  // the ranking area is reused as the staging ring
+  return v;
+}
+
 template <typename E, int D, bool GATHERED>
 __global__ void __launch_bounds__(kWideBlock) stage1_fused_kernel(Stage1Args a) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int wide_blocks = a.vnode_count * a.hkv;
   if ((int)blockIdx.x < wide_blocks) {
-    const int local_vnode = blockIdx.x / a.hkv;
-    wide_block<E, D, GATHERED>(a, smem, local_vnode, blockIdx.x - local_vnode * a.hkv);
+    const int rank = blockIdx.x / a.hkv;
+    const int local_vnode = wide_vnode_of_rank<GATHERED>(a, smem, rank);
+    wide_block<E, D, GATHERED>(a, smem, local_vnode, blockIdx.x - rank * a.hkv);
   } else {
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int item = (blockIdx.x - wide_blocks) * kWideWaves + wave;
     if (item >= a.narrow_count * a.hkv) return;  // whole wave; no block barrier below
     const int local_vnode = item / a.hkv;
     const int kvh = item - local_vnode * a.hkv;
     FT_TIME(unsigned long long t_start = FT_CLOCK(); unsigned long long rt_start = wall_clock64();)
-    const VnodeView vn = load_vnode<GATHERED>(a, a.narrow_begin + local_vnode);
-    const int rows_total = vn.q_len * a.g;
-    for (int row0 = 0; row0 < rows_total; row0 += 16) {
-      WaveState<D, 1> st;
-      // (the gathered baseline streams long contiguous runs: one tile in flight is enough there)
-      wave_attend<E, D, 1, GATHERED, !GATHERED>(a, vn, kvh, row0, 0, 1, smem + wave * TileGeom<D>::kBytes, st);
-      write_partials<D, 1>(a, vn, kvh, row0, st);
-    }
+    narrow_wave<E, D, GATHERED>(a, smem, wave, a.narrow_begin + local_vnode, kvh);
     FT_TIME(if (g_timing && (threadIdx.x & 63) == 0) {
       unsigned long long* out = g_timing + ((size_t)blockIdx.x * kWideWaves + wave) * 8;
       out[4] = FT_CLOCK() - t_start; out[5] = 0; out[6] = rt_start; out[7] = wall_clock64();
@@ -1006,8 +1238,8 @@ int launch_stage1_inst(const Stage1Args& a, int hkv, hipStream_t stream) {
 
 template <typename E, int D, bool GATHERED>
 int launch_stage1_fused(const Stage1Args& a, hipStream_t stream) {
-  constexpr size_t kWideLds = 2 * (size_t)WideGeom<D>::kBytes;
-  constexpr size_t kNarrowLds = (size_t)kWideWaves * TileGeom<D>::kBytes;
+  constexpr size_t kWideLds = (size_t)WideGeom<D>::kLds;
+  constexpr size_t kNarrowLds = (size_t)kWideWaves * NarrowGeom<D>::kLds;
   constexpr size_t lds = kWideLds > kNarrowLds ? kWideLds : kNarrowLds;
   auto kern = stage1_fused_kernel<E, D, GATHERED>;
   static bool configured = false;  // raising the dynamic LDS limit is idempotent
@@ -1098,6 +1330,9 @@ int check_common(int d, int g, int dtype) {
 extern "C" int ft_debug_set_timing(unsigned long long* buf) {
   return hipMemcpyToSymbol(HIP_SYMBOL(g_timing), &buf, sizeof(buf)) == hipSuccess ? 0 : -1;
 }
+extern "C" int ft_debug_set_timing_steps(int on) {
+  return hipMemcpyToSymbol(HIP_SYMBOL(g_timing_steps), &on, sizeof(on)) == hipSuccess ? 0 : -1;
+}
 #endif
 
 extern "C" {
@@ -1132,6 +1367,8 @@ static int stage1_setup(Stage1Args& a, const void* q, const void* k, const void*
       !vnode_to_q_offs || !vnode_to_q_lens || !mid_o || !mid_lse)
     return FT_ERR_NULL_POINTER;
   if (num_kv_heads < 1 || num_kv_heads > 65535 || !(sm_scale > 0.f)) return FT_ERR_ARGUMENT;
+  // the kernels form row addresses as slot * (32-bit byte stride)
+  if (sk0 < 0 || sv0 < 0 || sk0 >= (int64_t(1) << 31) || sv0 >= (int64_t(1) << 31)) return FT_ERR_ARGUMENT;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(mid_o) || (sq0 | sq1 | sk0 | sk1 | sv0 | sv1) % 8 != 0 ||
       (so0 | so1) % 4 != 0)
     return FT_ERR_ALIGNMENT;

@@ -12,7 +12,8 @@
  *   - dtype: FT_DTYPE_F16 or FT_DTYPE_BF16, the element type of q, k, v and o.
  *   - q, o:  [batch, Hq, D]; k, v: [slots, Hkv, D]; the last dimension is contiguous,
  *     the two outer strides are given in elements and must be multiples of 8, and the
- *     base pointers must be 16-byte aligned.  K and V are separate allocations.
+ *     base pointers must be 16-byte aligned.  K and V are separate allocations; their
+ *     slot strides must lie in [0, 2^31).
  *   - mid_o [rows, Hq, D] and mid_lse [rows, Hq] are caller-owned fp32 scratch; stage 1
  *     overwrites them with the per-vnode partial result normalised by its own soft-max
  *     sum and with log-sum-exp of the scaled scores (natural log).  mid_o strides must
