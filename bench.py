@@ -15,7 +15,8 @@ Prints ONE JSON line on stdout:
                (triton.testing.do_bench, kernel_bench/benchmark.py:59) with a larger flush.
   ms_per_step  wall clock of exactly --steps back-to-back calls / steps (warm caches,
                launch overhead included).
-  roofline     the dominant kernel of the call, timed live per launch with events.
+  roofline     the dominant kernel of the call; its duration is the mean over the timed steps
+               of the event-to-event time around its launch.
   cpu_baseline the reference's no-sharing formulation (per-request gathered KV, PyTorch
                ops) on this box's host cores, on a bounded sample of requests.
 """
@@ -157,6 +158,19 @@ def main():
     def step():
         fasttree_decode(inp.Q, inp.K_pool, inp.V_pool, o, *aux, prob["q_tiles"], prob["kv_tiles"], scale)
 
+    nums, offs = list(aux[11]), list(aux[12])
+
+    def stage1():
+        fasttree_decode_stage1(inp.Q, inp.K_pool, inp.V_pool, *aux[:6], scale, aux[9], aux[10], nums, offs,
+                               prob["q_tiles"], prob["kv_tiles"])
+
+    def stage2():
+        fasttree_decode_stage2(aux[6], aux[7], aux[8], aux[9], aux[10], o)
+
+    # The timed region: exactly --steps decode calls back to back.  It is run twice: once bare
+    # for the wall clock, once more as its two launches (what ft_decode enqueues) with an event on
+    # the launch stream before, between and after, for the per-kernel durations -- the events
+    # themselves cost a few microseconds per step, which must not leak into ms_per_step.
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -165,8 +179,14 @@ def main():
         step()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    for m in marks:
+        m[0].record(); stage1(); m[1].record(); stage2(); m[2].record()
+    torch.cuda.synchronize()
+    per_launch = {"stage1": statistics.mean(m[0].elapsed_time(m[1]) for m in marks) * 1e3,
+                  "stage2": statistics.mean(m[1].elapsed_time(m[2]) for m in marks) * 1e3}
     if args.profile_only:
-        log(f"profile-only: {args.steps} steps, {wall_ms * 1e3:.1f} us/step wall")
+        log(f"profile-only: {args.steps} steps, {wall_ms * 1e3:.1f} us/step wall, launches {per_launch}")
         return
 
     # ---- parity of this very run against the CPU oracle on a request sample
@@ -194,23 +214,6 @@ def main():
     cold_med, cold_p20, cold_p80 = quantiles(cold)
     warm_med, _, _ = quantiles(warm)
 
-    # ---- per-launch durations (cold), same events, one launch at a time
-    nums, offs = list(aux[11]), list(aux[12])
-    launches = {}
-
-    def timed(name, fn):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(); fn(); e1.record()
-        e1.synchronize()
-        launches.setdefault(name, []).append(e0.elapsed_time(e1) * 1e3)
-
-    for _ in range(reps):
-        flush.zero_()
-        timed("stage1", lambda: fasttree_decode_stage1(
-            inp.Q, inp.K_pool, inp.V_pool, *aux[:6], scale, aux[9], aux[10], nums, offs,
-            prob["q_tiles"], prob["kv_tiles"]))
-        timed("stage2", lambda: fasttree_decode_stage2(aux[6], aux[7], aux[8], aux[9], aux[10], o))
-    per_launch = {k: statistics.mean(v) for k, v in launches.items()}
     dominant = max(per_launch, key=per_launch.get)
 
     # algorithmic work of the stage-1 launch (both phases run in one kernel): every unique KV

@@ -1,0 +1,365 @@
+"""SGLang v0.2.13 decode hook on top of the HIP kernels.
+
+Mirrors the reference plugin ``fasttree_sglang_plugin_v0_2_13``:
+
+* ``FastTreeMetadata``          -- metadata.py:5-66 (pre-allocated device buffers, same
+  constructor arguments, defaults and attribute names);
+* ``decode_forward_fasttree``   -- plugin.py:15-51 (the body bound to
+  ``RadixAttention.decode_forward``);
+* ``prepare_for_fasttree_meta`` / ``prepare_for_fasttree_step`` -- schedule.py:12-283 (the
+  per-batch planner over the radix cache and the in-place ``kv_len += 1`` between decode steps);
+* ``load_fasttree_plugin``      -- plugin.py:234-238.
+
+Nothing here imports sglang at module import time.  The hook and the planner only use the
+attributes of the objects they are handed (duck typing), so they run against SGLang's own
+``RadixAttention`` / ``InputMetadata`` / ``ScheduleBatch`` / ``TreeNode`` and against any object
+with the same fields.
+"""
+
+from __future__ import annotations
+
+from collections import defaultdict, deque
+from types import MethodType
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+
+class FastTreeMetadata:
+    """Planner hyper-parameters plus the device buffers one decode step reads (metadata.py:5-66).
+
+    Buffers are allocated once at their maxima; a plan fills prefixes of them.  The defaults are
+    the reference's, including ``para_threshs1=(132, 132)`` / ``para_threshs2=(132, 528)``.
+    On MI355X pass ``TSQs=(256 // g, 16 // g)`` and thresholds scaled to 256 compute units.
+    """
+
+    def __init__(
+        self,
+        num_qo_heads: int,
+        num_kv_heads: int,
+        head_dim: int,
+        device="cuda",
+        alpha: float = 0.6,
+        beta: float = 0.3,
+        gamma: float = 0.1,
+        TSQs: Optional[Tuple[int, int]] = None,
+        TSKs: Tuple[int, int] = (32, 32),
+        kv_split_sizes: Tuple[int, int] = (1024, 128),
+        para_threshs1: Tuple[int, int] = (132, 132),
+        para_threshs2: Tuple[int, int] = (132, 528),
+        max_vnodes: int = 16384,
+        max_vnode_to_q_entries: int = 81920,
+        max_batch_size: int = 8192,
+    ):
+        self.num_qo_heads = num_qo_heads
+        self.num_kv_heads = num_kv_heads
+        self.head_dim = head_dim
+        self.kv_group_num = num_qo_heads // num_kv_heads
+        self.device = device
+        self.alpha, self.beta, self.gamma = alpha, beta, gamma
+        self.TSQs = TSQs if TSQs is not None else (64 // self.kv_group_num, 16 // self.kv_group_num)
+        self.TSKs = TSKs
+        self.kv_split_sizes = kv_split_sizes
+        self.para_threshs1 = para_threshs1
+        self.para_threshs2 = para_threshs2
+
+        def ints(n):
+            return torch.empty(n, dtype=torch.int32, device=device)
+
+        self.vnode_to_q_entries = ints(max_vnode_to_q_entries)
+        self.vnode_to_q_offs = ints(max_vnodes)
+        self.vnode_to_q_lens = ints(max_vnodes)
+        self.vnode_to_kv_offs = ints(max_vnodes)
+        self.vnode_to_kv_lens = ints(max_vnodes)
+        self.req_to_vnode_entries = ints(max_vnode_to_q_entries)
+        self.req_to_vnode_offs = ints(max_batch_size)
+        self.req_to_vnode_lens = ints(max_batch_size)
+        self.mid_o = torch.empty((max_vnode_to_q_entries, num_qo_heads, head_dim), dtype=torch.float32, device=device)
+        self.mid_lse = torch.empty((max_vnode_to_q_entries, num_qo_heads), dtype=torch.float32, device=device)
+
+        self.phase_node_nums: Optional[Sequence[int]] = None
+        self.phase_node_offsets: Optional[Sequence[int]] = None
+        self.phase_q_tile_sizes: Optional[Sequence[int]] = None
+        self.phase_kv_tile_sizes: Optional[Sequence[int]] = None
+        self.req_last_vnodes: Optional[List[int]] = None
+
+        print("FastTreeMetadata initialized")
+
+
+# ---------------------------------------------------------------------------------------
+# The hook body
+# ---------------------------------------------------------------------------------------
+def decode_forward_fasttree(self, q, k, v, input_metadata):
+    """``RadixAttention.decode_forward`` replacement (plugin.py:15-51).
+
+    Stores the step's K/V rows through the layer's own ``store_kv_cache``, then runs the tree
+    decode with the pool buffers, ``req_to_token`` as the flat KV-index array and the metadata
+    bound to ``input_metadata.fasttree``.  The output shape for ``qk_head_dim != v_head_dim``
+    follows the reference literally (plugin.py:22-23).
+    """
+    from .decode import fasttree_decode
+
+    if self.qk_head_dim != self.v_head_dim:
+        o = q.new_empty((q.shape[-1], self.tp_q_head_num * self.v_head_dim))
+    else:
+        o = torch.empty_like(q)
+    self.store_kv_cache(k, v, input_metadata)
+
+    meta = input_metadata.fasttree
+    fasttree_decode(
+        q.view(-1, self.tp_q_head_num, self.qk_head_dim),
+        input_metadata.token_to_kv_pool.get_key_buffer(self.layer_id),
+        input_metadata.token_to_kv_pool.get_value_buffer(self.layer_id),
+        o.view(-1, self.tp_q_head_num, self.v_head_dim),
+        input_metadata.req_to_token_pool.req_to_token,
+        meta.vnode_to_kv_offs, meta.vnode_to_kv_lens,
+        meta.vnode_to_q_entries, meta.vnode_to_q_offs, meta.vnode_to_q_lens,
+        meta.req_to_vnode_entries, meta.req_to_vnode_offs, meta.req_to_vnode_lens,
+        meta.mid_o, meta.mid_lse,
+        meta.phase_node_nums, meta.phase_node_offsets,
+        meta.phase_q_tile_sizes, meta.phase_kv_tile_sizes,
+        sm_scale=self.scaling,
+        logit_cap=self.logit_cap,
+    )
+    return o
+
+
+# ---------------------------------------------------------------------------------------
+# The per-batch planner over the radix cache
+# ---------------------------------------------------------------------------------------
+def _requests_per_radix_node(batch) -> Dict[object, List[int]]:
+    """Walks every request's token sequence (prompt, then generated tokens) down the radix tree
+    and lists, per node reached, the batch positions of the requests (schedule.py:18-35)."""
+    reqs_of = defaultdict(list)
+    for rid, req in enumerate(batch.reqs):
+        tokens_in, tokens_out = req.origin_input_ids, req.output_ids
+        total = len(tokens_in) + len(tokens_out)
+        node, pos = batch.tree_cache.root_node, 0
+        while pos < total:
+            token = tokens_in[pos] if pos < len(tokens_in) else tokens_out[pos - len(tokens_in)]
+            child = node.children.get(token)
+            if not child:
+                break
+            reqs_of[child].append(rid)
+            node = child
+            pos += len(child.key)
+    return reqs_of
+
+
+def prepare_for_fasttree_meta(batch, fasttree_metadata: FastTreeMetadata):
+    """Plans one decode batch (schedule.py:12-277) and binds the metadata to it.
+
+    As shipped, the reference's merge loop never takes a decision: it iterates
+    ``enumerate(node.children.values())`` (schedule.py:96), whose tuples are never keys of the
+    request map, so every radix node keeps its own vnodes (assignment 0 everywhere).  That is
+    the behaviour restated here; the cost model is therefore not evaluated.  Other literal
+    traits kept: the kv-split "reduction" of the first adaptation pass assigns a value to
+    itself (schedule.py:126), the second pass sets the KV tile sizes from the already replaced
+    query tile list (schedule.py:137-141), and parallelism counts KV *tiles*, not splits
+    (schedule.py:113).
+    """
+    meta = fasttree_metadata
+    root = batch.tree_cache.root_node
+    reqs_of = _requests_per_radix_node(batch)
+
+    # live nodes in BFS order with the offset of their first token along the path
+    order, token_offset = [], []
+    todo = deque([(root, 0)])
+    while todo:
+        node, off = todo.popleft()
+        order.append(node)
+        token_offset.append(off)
+        for child in node.children.values():
+            if child in reqs_of:
+                todo.append((child, off + len(node.value)))
+
+    n_reqs = [len(reqs_of[node]) if node in reqs_of else 0 for node in order]
+    seqlens = [len(node.value) for node in order]
+
+    q_tiles = meta.TSQs
+    kv_tiles = meta.TSKs
+    kv_splits = [meta.kv_split_sizes[0], meta.kv_split_sizes[0]]
+
+    def parallelism():
+        p = [0, 0]
+        for nq, length in zip(n_reqs, seqlens):
+            if nq > 0:
+                phase = 0 if nq > q_tiles[1] else 1
+                p[phase] += ((nq - 1) // q_tiles[phase] + 1) * ((length - 1) // kv_tiles[phase] + 1)
+        return [x * meta.num_kv_heads for x in p]
+
+    for it in range(3):
+        p = parallelism()
+        if it == 0:
+            low = [ph for ph in range(2) if 0 < p[ph] < meta.para_threshs1[ph]]
+            for ph in low:
+                kv_splits[ph] = kv_splits[1]
+            if not low:
+                break
+        elif it == 1:
+            if 0 < p[0] < meta.para_threshs2[0]:
+                q_tiles = [q_tiles[1], q_tiles[1]]
+                kv_tiles = [q_tiles[1], q_tiles[1]]
+            elif 0 < p[1] < meta.para_threshs2[1]:
+                q_tiles = [q_tiles[0], q_tiles[0]]
+                kv_tiles = [q_tiles[0], q_tiles[0]]
+            else:
+                break
+    meta.phase_q_tile_sizes = q_tiles
+    meta.phase_kv_tile_sizes = kv_tiles
+
+    kv_offs, kv_lens, q_entries, q_offs, q_lens = [], [], [], [], []
+    rows = batch.req_pool_indices.cpu()
+    stride = batch.req_to_token_pool.req_to_token.stride(0)
+
+    def emit(kv_start, length, members, q_tile, kv_split, n_q):
+        # one copy of the member list per KV split, cut into query tiles
+        for kv0 in range(0, length, kv_split):
+            q0 = len(q_entries)
+            q_entries.extend(members)
+            for s in range(0, n_q, q_tile):
+                kv_offs.append(kv_start + kv0)
+                kv_lens.append(min(kv0 + kv_split, length) - kv0)
+                q_offs.append(q0 + s)
+                q_lens.append(min(s + q_tile, n_q) - s)
+
+    for node, nq, length, off in zip(order, n_reqs, seqlens, token_offset):
+        if nq == 0:
+            continue
+        # the members are listed child by child where the node has live children (all of them
+        # keep assignment 0), else from the node itself; the KV is read through the row of the
+        # first member
+        groups = [c for c in node.children.values() if c in reqs_of] or [node]
+        members = [r for grp in groups for r in reqs_of[grp]]
+        phase = 0 if nq > q_tiles[1] else 1
+        emit(stride * int(rows[members[0]]) + off, length, members, q_tiles[phase], kv_splits[phase], nq)
+
+    # generated tokens: one chain of single-request vnodes per request, after the tree's
+    last = [0] * len(batch.reqs)
+    for rid, req in enumerate(batch.reqs):
+        prefix = len(req.origin_input_ids)
+        emit(stride * int(rows[rid]) + prefix, len(req.output_ids) + 1, [rid], 1, kv_splits[1], 1)
+        last[rid] = len(kv_lens) - 1  # unchanged by the reordering below
+    meta.req_last_vnodes = last
+
+    per_req = [[] for _ in batch.reqs]
+    for row, r in enumerate(q_entries):
+        per_req[r].append(row)
+    req_offs, req_lens, acc = [], [], 0
+    for lst in per_req:
+        req_offs.append(acc)
+        req_lens.append(len(lst))
+        acc += len(lst)
+    req_entries = [row for lst in per_req for row in lst]
+
+    above = [i for i, n in enumerate(q_lens) if n > q_tiles[1]]
+    below = [i for i, n in enumerate(q_lens) if n <= q_tiles[1]]
+    perm = above + below
+    meta.phase_node_nums = [len(above), len(below)]
+    meta.phase_node_offsets = [0, len(above)]
+
+    def upload(dst, values):
+        src = torch.tensor(values, device="cpu", dtype=torch.int32)
+        dst[: src.numel()].copy_(src, non_blocking=True)
+
+    upload(meta.vnode_to_q_entries, q_entries)
+    upload(meta.vnode_to_q_offs, [q_offs[i] for i in perm])
+    upload(meta.vnode_to_q_lens, [q_lens[i] for i in perm])
+    upload(meta.vnode_to_kv_offs, [kv_offs[i] for i in perm])
+    upload(meta.vnode_to_kv_lens, [kv_lens[i] for i in perm])
+    upload(meta.req_to_vnode_entries, req_entries)
+    upload(meta.req_to_vnode_offs, req_offs)
+    upload(meta.req_to_vnode_lens, req_lens)
+
+    batch.fasttree_metadata = meta
+
+
+def prepare_for_fasttree_step(batch, fasttree_metadata: FastTreeMetadata):
+    """Between two decode steps of an unchanged batch every request has one more token: its
+    last vnode grows by one, on the device (schedule.py:280-283)."""
+    bs = len(batch.reqs)
+    one = torch.ones(bs, device=fasttree_metadata.device, dtype=torch.int32)
+    fasttree_metadata.vnode_to_kv_lens[fasttree_metadata.req_last_vnodes] += one
+
+
+# ---------------------------------------------------------------------------------------
+# Loader
+# ---------------------------------------------------------------------------------------
+def load_fasttree_plugin(enable_fasttree=True, annotate_breakdown=False):
+    """Installs the hook into SGLang v0.2.13 (plugin.py:234-238).
+
+    With the reference's plugin package importable, its loader is used unchanged with the
+    kernel entry point, the metadata class and the planner swapped for the ones in this module.
+    Without it, the three patches are applied here: ``RadixAttention.decode_forward``,
+    ``InputMetadata.from_schedule_batch`` (carries ``batch.fasttree_metadata``), and
+    ``ModelTpServer`` (metadata creation; a fresh plan when the batch changed, the ``+1`` step
+    otherwise, before every decode forward).  Raises ImportError when sglang is not installed.
+    """
+    if not enable_fasttree and not annotate_breakdown:
+        print("[Warning] FastTree plugin is not enabled")
+        return
+    import sys
+
+    from .decode import fasttree_decode
+
+    this = sys.modules[__name__]
+    try:
+        import fasttree_sglang_plugin_v0_2_13.plugin as ref_plugin
+        import fasttree_sglang_plugin_v0_2_13.schedule as ref_schedule
+    except ImportError:
+        ref_plugin = None
+    if ref_plugin is not None:
+        ref_plugin.fasttree_decode = fasttree_decode
+        ref_plugin.FastTreeMetadata = FastTreeMetadata
+        ref_schedule.prepare_for_fasttree_meta = this.prepare_for_fasttree_meta
+        ref_schedule.prepare_for_fasttree_step = this.prepare_for_fasttree_step
+        return ref_plugin.load_fasttree_plugin(enable_fasttree, annotate_breakdown)
+
+    from sglang.srt.layers.radix_attention import RadixAttention
+    from sglang.srt.managers.tp_worker import ModelTpServer
+    from sglang.srt.model_executor.forward_batch_info import InputMetadata
+
+    if not enable_fasttree:
+        return
+
+    radix_init = RadixAttention.__init__
+
+    def radix_init_with_hook(self, *args, **kwargs):
+        radix_init(self, *args, **kwargs)
+        self.decode_forward = MethodType(decode_forward_fasttree, self)
+
+    RadixAttention.__init__ = radix_init_with_hook
+
+    meta_from_batch = InputMetadata.from_schedule_batch.__func__
+
+    def meta_from_batch_with_plan(cls, model_runner, batch, forward_mode):
+        ret = meta_from_batch(cls, model_runner, batch, forward_mode)
+        ret.fasttree = getattr(batch, "fasttree_metadata", None)
+        return ret
+
+    InputMetadata.from_schedule_batch = classmethod(meta_from_batch_with_plan)
+
+    server_init = ModelTpServer.__init__
+
+    def server_init_with_metadata(self, gpu_id, tp_rank, server_args, nccl_port, model_overide_args):
+        server_args.disable_cuda_graph = True  # plugin.py:209-211
+        server_init(self, gpu_id, tp_rank, server_args, nccl_port, model_overide_args)
+        self.fasttree_metadata = FastTreeMetadata(
+            self.model_config.num_attention_heads, self.model_config.num_key_value_heads,
+            self.model_config.head_dim, torch.device("cuda", self.gpu_id))
+        self._fasttree_planned_for = None
+
+    ModelTpServer.__init__ = server_init_with_metadata
+
+    decode_batch = ModelTpServer.forward_decode_batch
+
+    def decode_batch_with_plan(self, batch):
+        members = tuple(id(r) for r in batch.reqs)
+        if self._fasttree_planned_for == members:
+            prepare_for_fasttree_step(batch, self.fasttree_metadata)
+        else:
+            prepare_for_fasttree_meta(batch, self.fasttree_metadata)
+            self._fasttree_planned_for = members
+        return decode_batch(self, batch)
+
+    ModelTpServer.forward_decode_batch = decode_batch_with_plan

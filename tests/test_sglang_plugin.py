@@ -1,0 +1,253 @@
+"""The SGLang hook mirror: planner over a radix cache (CPU) and the hook body (GPU).
+
+The reference's plugin imports sglang at module level (schedule.py:6-7, plugin.py:2), which is
+not installed here, so no golden vectors exist for this planner: the first test is a
+known-answer case derived by hand from schedule.py:12-277, the others check the invariants any
+correct plan has (every token of every request is covered by exactly one of the request's
+scratch rows).  Parity of the array *order* beyond the hand case is unpinned.
+"""
+import math
+import random
+
+import pytest
+import torch
+
+from fasttree_hip.sglang_plugin import (FastTreeMetadata, decode_forward_fasttree, prepare_for_fasttree_meta,
+                                        prepare_for_fasttree_step)
+
+
+# ---- stand-ins with the fields of SGLang's TreeNode / Req / ScheduleBatch / pools
+class Node:
+    def __init__(self, key=(), value=()):
+        self.key, self.value, self.children = list(key), list(value), {}
+
+
+class Req:
+    def __init__(self, origin_input_ids, output_ids):
+        self.origin_input_ids, self.output_ids = list(origin_input_ids), list(output_ids)
+
+
+class Obj:
+    def __init__(self, **kw):
+        self.__dict__.update(kw)
+
+
+def insert(root, tokens, slots):
+    """Radix insert without node splitting: callers insert shared prefixes first."""
+    node, pos = root, 0
+    while pos < len(tokens):
+        child = node.children.get(tokens[pos])
+        if child is None:
+            child = Node(tokens[pos:], slots[pos:])
+            node.children[tokens[pos]] = child
+            return
+        assert tokens[pos:pos + len(child.key)] == child.key
+        node, pos = child, pos + len(child.key)
+
+
+def make_batch(prompts, outputs, shared_prefixes, device="cpu", max_ctx=64, row_of=None):
+    """prompts[r]: token ids; shared_prefixes: token lists inserted first as their own nodes.
+    Pool slots are handed out so that shared prefixes own the same slots in every row."""
+    root = Node()
+    slot_of_prefix = {}
+    next_slot = [1]
+
+    def slots_for(tokens):
+        out = []
+        for i in range(len(tokens)):
+            key = tuple(tokens[: i + 1])
+            if key not in slot_of_prefix:
+                slot_of_prefix[key] = next_slot[0]
+                next_slot[0] += 1
+            out.append(slot_of_prefix[key])
+        return out
+
+    for pre in shared_prefixes:
+        insert(root, pre, slots_for(pre))
+    for p in prompts:
+        insert(root, p, slots_for(p))
+    n = len(prompts)
+    row_of = row_of or list(range(n))
+    req_to_token = torch.zeros((max(row_of) + 1, max_ctx), dtype=torch.int32)
+    for r, (p, out) in enumerate(zip(prompts, outputs)):
+        sl = slots_for(p)
+        gen = list(range(next_slot[0], next_slot[0] + len(out) + 1))  # generated tokens + the one being decoded
+        next_slot[0] += len(out) + 1
+        req_to_token[row_of[r], : len(sl) + len(gen)] = torch.tensor(sl + gen, dtype=torch.int32)
+    batch = Obj(reqs=[Req(p, o) for p, o in zip(prompts, outputs)], tree_cache=Obj(root_node=root),
+                req_pool_indices=torch.tensor(row_of, dtype=torch.int64, device=device),
+                req_to_token_pool=Obj(req_to_token=req_to_token.to(device)))
+    return batch, next_slot[0]
+
+
+def plan_lists(meta, batch):
+    nv = sum(meta.phase_node_nums)
+    rows = int(meta.req_to_vnode_offs[len(batch.reqs) - 1] + meta.req_to_vnode_lens[len(batch.reqs) - 1])
+    return dict(kv_offs=meta.vnode_to_kv_offs[:nv].tolist(), kv_lens=meta.vnode_to_kv_lens[:nv].tolist(),
+                q_offs=meta.vnode_to_q_offs[:nv].tolist(), q_lens=meta.vnode_to_q_lens[:nv].tolist(),
+                q_entries=meta.vnode_to_q_entries[:rows].tolist(), req_entries=meta.req_to_vnode_entries[:rows].tolist(),
+                req_offs=meta.req_to_vnode_offs[: len(batch.reqs)].tolist(),
+                req_lens=meta.req_to_vnode_lens[: len(batch.reqs)].tolist())
+
+
+def small_meta(device="cpu", hq=32, hkv=8, d=128, **kw):
+    return FastTreeMetadata(hq, hkv, d, device=device, max_vnodes=4096, max_vnode_to_q_entries=8192,
+                            max_batch_size=512, **kw)
+
+
+def test_metadata_defaults_follow_the_reference():
+    m = small_meta()
+    assert m.kv_group_num == 4 and m.TSQs == (16, 4) and m.TSKs == (32, 32)
+    assert m.kv_split_sizes == (1024, 128) and m.para_threshs1 == (132, 132) and m.para_threshs2 == (132, 528)
+    assert (m.alpha, m.beta, m.gamma) == (0.6, 0.3, 0.1)
+    assert m.mid_o.shape == (8192, 32, 128) and m.mid_o.dtype == torch.float32
+    assert m.mid_lse.shape == (8192, 32)
+    for t in (m.vnode_to_q_entries, m.vnode_to_q_offs, m.vnode_to_kv_lens, m.req_to_vnode_entries, m.req_to_vnode_offs):
+        assert t.dtype == torch.int32
+    assert FastTreeMetadata(64, 8, 128, device="cpu", max_vnodes=8, max_vnode_to_q_entries=8, max_batch_size=8).TSQs == (8, 2)
+
+
+def test_hand_derived_plan():
+    # radix tree: A=[1,2,3,4] -> B=[5,6] (request 0), C=[7,8,9] (requests 1, 2)
+    prompts = [[1, 2, 3, 4, 5, 6], [1, 2, 3, 4, 7, 8, 9], [1, 2, 3, 4, 7, 8, 9]]
+    outputs = [[10, 11], [12], []]
+    batch, _ = make_batch(prompts, outputs, shared_prefixes=[[1, 2, 3, 4]], row_of=[2, 0, 5])
+    meta = small_meta()
+    prepare_for_fasttree_meta(batch, meta)
+    s = 64  # row stride of req_to_token
+    # parallelism [0, 24] < thresholds: pass 0 leaves the splits, pass 1 takes its second branch
+    assert list(meta.phase_q_tile_sizes) == [16, 16] and list(meta.phase_kv_tile_sizes) == [16, 16]
+    assert list(meta.phase_node_nums) == [0, 6] and list(meta.phase_node_offsets) == [0, 0]
+    got = plan_lists(meta, batch)
+    assert got["kv_offs"] == [2 * s + 0, 2 * s + 4, 0 * s + 4, 2 * s + 6, 0 * s + 7, 5 * s + 7]
+    assert got["kv_lens"] == [4, 2, 3, 3, 2, 1]
+    assert got["q_offs"] == [0, 3, 4, 6, 7, 8]
+    assert got["q_lens"] == [3, 1, 2, 1, 1, 1]
+    assert got["q_entries"] == [0, 1, 2, 0, 1, 2, 0, 1, 2]
+    assert got["req_entries"] == [0, 3, 6, 1, 4, 7, 2, 5, 8]
+    assert got["req_offs"] == [0, 3, 6] and got["req_lens"] == [3, 3, 3]
+    assert meta.req_last_vnodes == [3, 4, 5]
+    assert batch.fasttree_metadata is meta
+    prepare_for_fasttree_step(batch, meta)
+    assert meta.vnode_to_kv_lens[:6].tolist() == [4, 2, 3, 4, 3, 2]
+
+
+def covered_slots(meta, batch):
+    """Per request: the multiset of pool slots its scratch rows attend to."""
+    flat = batch.req_to_token_pool.req_to_token.reshape(-1).cpu()
+    got = plan_lists(meta, batch)
+    out = [[] for _ in batch.reqs]
+    for kv_off, kv_len, q_off, q_len in zip(got["kv_offs"], got["kv_lens"], got["q_offs"], got["q_lens"]):
+        for r in got["q_entries"][q_off:q_off + q_len]:
+            out[r] += flat[kv_off:kv_off + kv_len].tolist()
+    return out
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_every_token_is_covered_once(seed):
+    rng = random.Random(seed)
+    n_groups, per_group = rng.randint(1, 4), rng.randint(1, 24)
+    system = [rng.randint(1, 10**6) for _ in range(rng.randint(1, 40))]
+    prefixes, prompts, outputs = [system], [], []
+    for _ in range(n_groups):
+        mid = system + [rng.randint(1, 10**6) for _ in range(rng.randint(1, 30))]
+        prefixes.append(mid)
+        for _ in range(per_group):
+            prompts.append(mid + [rng.randint(1, 10**6) for _ in range(rng.randint(1, 12))])
+            outputs.append([rng.randint(1, 10**6) for _ in range(rng.randint(0, 5))])
+    batch, _ = make_batch(prompts, outputs, prefixes, max_ctx=128)
+    meta = small_meta(kv_split_sizes=(16, 8))
+    prepare_for_fasttree_meta(batch, meta)
+    cov = covered_slots(meta, batch)
+    table = batch.req_to_token_pool.req_to_token
+    for r, (p, o) in enumerate(zip(prompts, outputs)):
+        want = table[r, : len(p) + len(o) + 1].tolist()
+        assert sorted(cov[r]) == sorted(want)
+    got = plan_lists(meta, batch)
+    nv0 = meta.phase_node_nums[0]
+    assert all(n > meta.phase_q_tile_sizes[1] for n in got["q_lens"][:nv0])
+    assert all(n <= meta.phase_q_tile_sizes[1] for n in got["q_lens"][nv0:])
+    for r in range(len(prompts)):
+        rows = got["req_entries"][got["req_offs"][r]: got["req_offs"][r] + got["req_lens"][r]]
+        assert all(got["q_entries"][i] == r for i in rows) and rows == sorted(rows)
+
+
+# ---- the hook body on the GPU
+class FakeLayer:
+    def __init__(self, hq, hkv, d, layer_id=0):
+        self.tp_q_head_num, self.tp_k_head_num, self.qk_head_dim, self.v_head_dim = hq, hkv, d, d
+        self.layer_id, self.scaling, self.logit_cap = layer_id, 1.0 / math.sqrt(d), -1
+
+    def store_kv_cache(self, k, v, input_metadata):
+        pool = input_metadata.token_to_kv_pool
+        pool.k[self.layer_id][input_metadata.out_cache_loc] = k.view(-1, self.tp_k_head_num, self.qk_head_dim)
+        pool.v[self.layer_id][input_metadata.out_cache_loc] = v.view(-1, self.tp_k_head_num, self.v_head_dim)
+
+
+class FakePool:
+    def __init__(self, k, v):
+        self.k, self.v = [k], [v]
+
+    def get_key_buffer(self, layer_id):
+        return self.k[layer_id]
+
+    def get_value_buffer(self, layer_id):
+        return self.v[layer_id]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_hook_matches_dense_attention(device, dtype):
+    import fasttree_oracle as oracle
+    from helpers import assert_parity
+
+    rng = random.Random(7)
+    hq, hkv, d = 32, 8, 128
+    system = [rng.randint(1, 10**6) for _ in range(70)]
+    prefixes, prompts, outputs = [system], [], []
+    for _ in range(3):
+        mid = system + [rng.randint(1, 10**6) for _ in range(33)]
+        prefixes.append(mid)
+        for _ in range(9):
+            prompts.append(mid + [rng.randint(1, 10**6) for _ in range(rng.randint(1, 20))])
+            outputs.append([rng.randint(1, 10**6) for _ in range(rng.randint(0, 6))])
+    n = len(prompts)
+    rows = list(range(n))
+    rng.shuffle(rows)
+    batch, n_slots = make_batch(prompts, outputs, prefixes, device=device, max_ctx=256, row_of=rows)
+    meta = small_meta(device=device, TSQs=(256 // 4, 16 // 4))
+    prepare_for_fasttree_meta(batch, meta)
+
+    g = torch.Generator().manual_seed(3)
+    k_pool = torch.randn((n_slots + 8, hkv, d), generator=g).to(dtype).to(device)
+    v_pool = torch.randn((n_slots + 8, hkv, d), generator=g).to(dtype).to(device)
+    q = torch.randn((n, hq * d), generator=g).to(dtype).to(device)
+    k_new = torch.randn((n, hkv * d), generator=g).to(dtype).to(device)
+    v_new = torch.randn((n, hkv * d), generator=g).to(dtype).to(device)
+    table = batch.req_to_token_pool.req_to_token
+    lens = [len(p) + len(o) + 1 for p, o in zip(prompts, outputs)]
+    out_loc = torch.tensor([int(table[rows[r], lens[r] - 1]) for r in range(n)], device=device)
+    im = Obj(token_to_kv_pool=FakePool(k_pool, v_pool), req_to_token_pool=batch.req_to_token_pool,
+             fasttree=meta, out_cache_loc=out_loc)
+    layer = FakeLayer(hq, hkv, d)
+    layer.decode_forward = decode_forward_fasttree.__get__(layer)
+    o = layer.decode_forward(q, k_new, v_new, im)
+    torch.cuda.synchronize()
+    assert o.shape == q.shape and o.dtype == dtype
+    paths = [table[rows[r], : lens[r]].cpu().long() for r in range(n)]
+    want = oracle.dense_attention(q.view(n, hq, d).cpu(), k_pool.cpu(), v_pool.cpu(), paths, layer.scaling)
+    assert_parity(o.view(n, hq, d).cpu(), want, "hook", out_dtype=dtype)
+
+    # one more token per request: grow the last vnodes in place, as between two decode steps
+    for r in range(n):
+        table[rows[r], lens[r]] = n_slots + 0  # any valid slot; every request gets the same new row here
+    k_pool[n_slots] = torch.randn((hkv, d), generator=g).to(dtype).to(device)
+    v_pool[n_slots] = torch.randn((hkv, d), generator=g).to(dtype).to(device)
+    prepare_for_fasttree_step(batch, meta)
+    im.out_cache_loc = torch.full((n,), n_slots, device=device)
+    o2 = layer.decode_forward(q, k_pool[n_slots].reshape(1, -1).expand(n, -1).contiguous(),
+                              v_pool[n_slots].reshape(1, -1).expand(n, -1).contiguous(), im)
+    torch.cuda.synchronize()
+    paths2 = [table[rows[r], : lens[r] + 1].cpu().long() for r in range(n)]
+    want2 = oracle.dense_attention(q.view(n, hq, d).cpu(), k_pool.cpu(), v_pool.cpu(), paths2, layer.scaling)
+    assert_parity(o2.view(n, hq, d).cpu(), want2, "hook after step", out_dtype=dtype)
