@@ -40,6 +40,7 @@ MFMA_PEAK_TFLOPS = 2500.0      # dense fp16 / bf16
 
 WORKLOADS = {
     # name: (nodes per level, context per level, Hq, Hkv, dtype)
+    "c1": ([1, 16], [1024, 128], 32, 32, "fp16"),
     "c2": ([1, 64], [4096, 256], 32, 8, "fp16"),
     "c3": ([1, 10, 400], [4000, 400, 40], 32, 8, "fp16"),
     "c4": ([1, 2048], [512, 1024], 32, 8, "bf16"),
@@ -293,7 +294,7 @@ def main():
         "vs_baseline": None,
         "dtype": "f16" if prob["dtype"] == "fp16" else "bf16",
         "data": "synthetic",
-        "config": {"workload": {"c2": "2-level tree 1x4096 + 64x256", "c3": "3-level tree N=[1,10,400] C=[4000,400,40]",
+        "config": {"workload": {"c1": "2-level tree 1x1024 + 16x128", "c2": "2-level tree 1x4096 + 64x256", "c3": "3-level tree N=[1,10,400] C=[4000,400,40]",
                                 "c4": "2-level tree 1x512 + 2048x1024"}[args.workload]
                    + f", {prob['hq']}q/{prob['hkv']}kv heads, head_dim 128, {prob['dtype']}, paged pool (page 1, shuffled), "
                    + f"{prob['batch']} requests", "planner_preset": args.preset,

@@ -522,6 +522,12 @@ __device__ int g_timing_steps = 0;  // 1: report per-step phases (scores, soft-m
 #endif
 constexpr int kWideWaves = 8;
 constexpr int kWideBlock = kWave * kWideWaves;
+#ifndef FT_WIDE_BUFS
+#define FT_WIDE_BUFS 4
+#endif
+#ifndef FT_WIDE_IDX
+#define FT_WIDE_IDX 4096
+#endif
 
 // LDS layout of the wide kernel: rows of 2*D bytes back to back (no padding), 64-token super
 // tiles of two 32-token tiles, a ring of four buffers, then a staging area for the run's slot
@@ -535,16 +541,17 @@ template <int D> struct WideGeom {
   static constexpr int kChunks = D / 8;                  // 16-byte chunks per row
   static constexpr int kSub = 2;
   static constexpr int kTokens = kSub * kTileTokens;     // 64
-  static constexpr int kBufs = 4;
+  static constexpr int kBufs = FT_WIDE_BUFS;
+  static constexpr int kAhead = kBufs - 1;               // super tiles in flight beyond the current one
   static constexpr int kTileBytes = kTileTokens * kRowBytes;
   static constexpr int kBytesK = kTokens * kRowBytes;
   static constexpr int kBytes = 2 * kBytesK;             // K + V of one buffer
-  static constexpr int kRing = kBufs * kBytes;           // a power of two
+  static constexpr int kRing = kBufs * kBytes;
   static constexpr int kGroupRows = kWave / kChunks;     // rows per 1 KB load group
   static constexpr int kGroups = kTokens / kGroupRows;   // groups per matrix and super tile
   static constexpr int kUnits = 2 * kGroups / kWideWaves;                       // loads per wave and super tile
   static constexpr int kSlots = kGroups >= kWideWaves ? kGroups / kWideWaves : 1;  // distinct rows among them
-  static constexpr int kIdxCap = 4096;                   // slot indices staged at a time (tokens)
+  static constexpr int kIdxCap = FT_WIDE_IDX;             // slot indices staged at a time (tokens)
   static constexpr int kLds = kRing + 4 * kIdxCap;
   static __device__ __forceinline__ int swz(int row) { return (((row & 3) << 2) | ((row >> 2) & 3)) & (kChunks - 1); }
 };
@@ -589,8 +596,8 @@ __device__ __forceinline__ void load_q_frags32(const Stage1Args& a, const VnodeV
 // Per-lane LDS byte addresses of the operand reads inside tile 0 of the current buffer, for
 // contraction step / dim block 0.  Thanks to the XOR layout the address for step ks (dim block
 // db) is the base with 32*ks (64*db) XOR-ed in; the second tile of the super tile is a constant
-// offset away and the next buffer of the ring is kBytes further, modulo the ring size (the
-// dynamic LDS segment starts at 0).
+// offset away and buffer b of the ring is b * kBytes further (the dynamic LDS segment starts
+// at 0).
 struct WideLane {
   unsigned k;     // K operand: row lane%32, chunk lane/32 (step ks: chunk 2*ks + lane/32)
   unsigned v_lo;  // transposed V read: tokens 4*(lane/32) + 0..3 (+16 for u = 1), dims 0..31
@@ -609,12 +616,8 @@ __device__ __forceinline__ void init_lane(WideLane& la) {
   la.v_hi = W::kBytesK + row_hi * W::kRowBytes + 16 * (chunk ^ W::swz(row_hi)) + 8 * (p & 1);
 }
 
-template <int D>
-__device__ __forceinline__ void next_buffer(WideLane& la) {
-  using W = WideGeom<D>;
-  la.k = (la.k + W::kBytes) & (W::kRing - 1);
-  la.v_lo = (la.v_lo + W::kBytes) & (W::kRing - 1);
-  la.v_hi = (la.v_hi + W::kBytes) & (W::kRing - 1);
+__device__ __forceinline__ WideLane at_buffer(const WideLane& la0, unsigned buffer_offset) {
+  return WideLane{la0.k + buffer_offset, la0.v_lo + buffer_offset, la0.v_hi + buffer_offset};
 }
 
 // 16 bytes per lane from global memory straight into LDS at lds_base + 16 * lane (lds_base is
@@ -820,8 +823,9 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
     load_q_frags32<D, GATHERED>(a, vn, kvh, active ? my_row0 : rows_total, qf);
     WideState<D> st;
     reset_state<D>(st);
-    WideLane la;
-    init_lane<D>(la);
+    WideLane la0;
+    init_lane<D>(la0);
+    unsigned cur = 0;  // byte offset of the ring buffer that holds the current super tile
 
     // slot indices of tokens [idx_base, idx_base + kIdxCap) of the run, staged by the whole block
     int idx_base = 0;
@@ -838,7 +842,7 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
         __syncthreads();
       }
     };
-    // rows of super tile j -> ring buffer j % 4.  Tokens past the run repeat its last token: the
+    // rows of super tile j -> ring buffer j % kBufs.  Tokens past the run repeat its last token: the
     // scores of such rows are masked and their V rows are finite.
     auto issue_rows = [&](int j) {
       if (j >= nsuper) return;
@@ -848,7 +852,7 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
           stage_indices(idx_base + W::kIdxCap);
         }
       }
-      const unsigned buf = (unsigned)(j & (W::kBufs - 1)) * W::kBytes;
+      const unsigned buf = (unsigned)(j % W::kBufs) * W::kBytes;
       unsigned srow[W::kSlots];
       unsigned chunk[W::kSlots];
 #pragma unroll
@@ -873,23 +877,24 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
     // nothing the compiler itself tracks (the Q fragments) may still be in flight in the loop:
     // a wait for it there would also wait for every direct load
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    issue_rows(0);
-    issue_rows(1);
-    issue_rows(2);
+#pragma unroll
+    for (int j = 0; j < W::kAhead; ++j) issue_rows(j);
     FT_TIME(unsigned long long t_start = FT_CLOCK(); unsigned long long rt_start = wall_clock64(); unsigned long long t_wait = 0, t_bar = 0, t_issue = 0, t_comp = 0; unsigned long long t_step[4] = {0, 0, 0, 0};)
     for (int super = 0; super < nsuper; ++super) {
-      // publish super tile `super` to the block; the two after it may stay in flight
+      // publish super tile `super` to the block; the ones after it may stay in flight
       FT_TIME(unsigned long long c0 = FT_CLOCK();)
-      if (super + 2 < nsuper) wait_direct_loads<2 * W::kUnits>();
-      else if (super + 1 < nsuper) wait_direct_loads<W::kUnits>();
+      const int behind = min(nsuper - 1 - super, W::kAhead - 1);
+      if (behind >= 2) wait_direct_loads<2 * W::kUnits>();
+      else if (behind == 1) wait_direct_loads<W::kUnits>();
       else wait_direct_loads<0>();
       FT_TIME(unsigned long long c1 = FT_CLOCK();)
       __syncthreads();
       FT_TIME(unsigned long long c2 = FT_CLOCK();)
       // the buffer consumed before that barrier is free: refill it
-      issue_rows(super + 3);
+      issue_rows(super + W::kAhead);
       FT_TIME(unsigned long long c3 = FT_CLOCK();)
       if (active) {
+        const WideLane la = at_buffer(la0, cur);
 #pragma unroll 1
         for (int sub = 0; sub < W::kSub; ++sub) {
           const int tile = super * W::kSub + sub;
@@ -898,7 +903,7 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
           if (valid > 0) tile_step32<E, D>(la, sub * W::kTileBytes, valid, a.scale_log2, qf, st FT_TIME(, t_step));
         }
       }
-      next_buffer<D>(la);
+      cur = cur + W::kBytes == W::kRing ? 0u : cur + W::kBytes;
       FT_TIME(unsigned long long c4 = FT_CLOCK(); t_wait += c1 - c0; t_bar += c2 - c1; t_issue += c3 - c2; t_comp += c4 - c3;)
     }
     FT_TIME(if (g_timing && lane == 0) {
@@ -952,9 +957,6 @@ __device__ __forceinline__ void narrow_wave(const Stage1Args& a, char* smem, int
   const char* kbase = a.k + 2 * ((int64_t)kvh * a.sk1);
   const char* vbase = a.v + 2 * ((int64_t)kvh * a.sv1);
   const unsigned k_stride = (unsigned)(2 * a.sk0), v_stride = (unsigned)(2 * a.sv0);  // bytes, < 2^32 (checked by the host)
-  unsigned src_off[N::kGroups];
-#pragma unroll
-  for (int g = 0; g < N::kGroups; ++g) src_off[g] = 16 * (pos ^ N::swz(g * N::kGroupRows + grp_row));
 
   // operand read addresses: K row 16*tb + p, chunk c (contraction step ks: chunk 4*ks + c);
   // V tokens 4*c + p/4 (+16), chunk 2*db + (p%4)/2, half p%2
@@ -986,23 +988,19 @@ __device__ __forceinline__ void narrow_wave(const Stage1Args& a, char* smem, int
           wave_lds_fence();
         }
       };
-      // pool rows of the tokens this lane loads in `tile`; tokens past the run repeat its last
-      // token (their scores are masked, their V rows are finite)
-      unsigned srow[N::kGroups];
-      auto find_rows = [&](int tile) {
+      // K (or V) rows of `tile` -> the wave's K (V) tile.  Tokens past the run repeat its last
+      // token (their scores are masked, their V rows are finite).  The slot indices are read
+      // from the staged window each time rather than kept in registers between the two calls.
+      auto issue = [&](int tile, bool is_v) {
         if constexpr (!GATHERED) {
           if (tile * kTileTokens >= idx_base + N::kIdxCap) stage_indices(idx_base + N::kIdxCap);
         }
 #pragma unroll
         for (int g = 0; g < N::kGroups; ++g) {
-          const int t = min(tile * kTileTokens + g * N::kGroupRows + grp_row, vn.kv_len - 1);
-          srow[g] = GATHERED ? (unsigned)(vn.kv_base + t) : (unsigned)idx_lds[t - idx_base];
-        }
-      };
-      auto issue = [&](bool is_v) {
-#pragma unroll
-        for (int g = 0; g < N::kGroups; ++g) {
-          const char* src = (is_v ? vbase : kbase) + (uint64_t)srow[g] * (is_v ? v_stride : k_stride) + src_off[g];
+          const int row = g * N::kGroupRows + grp_row;
+          const int t = min(tile * kTileTokens + row, vn.kv_len - 1);
+          const unsigned srow = GATHERED ? (unsigned)(vn.kv_base + t) : (unsigned)idx_lds[t - idx_base];
+          const char* src = (is_v ? vbase : kbase) + (uint64_t)srow * (is_v ? v_stride : k_stride) + 16 * (pos ^ N::swz(row));
           load_direct16(src, lds0 + (is_v ? N::kBytesK : 0) + g * 1024);
         }
       };
@@ -1010,9 +1008,8 @@ __device__ __forceinline__ void narrow_wave(const Stage1Args& a, char* smem, int
       // nothing the compiler itself tracks may still be in flight below: a wait for it would
       // also wait for every direct load
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-      find_rows(0);
-      issue(false);
-      issue(true);
+      issue(0, false);
+      issue(0, true);
       for (int tile = 0; tile < ntiles; ++tile) {
         const bool more = tile + 1 < ntiles;
         const int valid = vn.kv_len - tile * kTileTokens;
@@ -1024,11 +1021,11 @@ __device__ __forceinline__ void narrow_wave(const Stage1Args& a, char* smem, int
           s[tb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks) s[tb] = E::mfma(lds_read16(k_addr[tb] ^ (64u * ks)), qf[0][ks], s[tb]);
+          __builtin_amdgcn_sched_barrier(0);  // one token block's operands at a time: keeps the register count low
         }
         if (more) {
-          find_rows(tile + 1);
           __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the K tile has been read
-          issue(false);
+          issue(tile + 1, false);
         }
         if (valid < kTileTokens) {
 #pragma unroll
@@ -1074,13 +1071,23 @@ __device__ __forceinline__ void narrow_wave(const Stage1Args& a, char* smem, int
         }
         if (more) {
           __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the V tile has been read
-          issue(true);
+          issue(tile + 1, true);
         }
       }
     }
     finish_state<D, 1>(st);
     write_partials<D, 1>(a, vn, kvh, row0, st);
   }
+}
+
+// Narrow vnodes alone (a launch without wide vnodes), one wave per block: the footprint of one
+// LDS tile instead of a wide block's ring, so that more of these latency-bound waves share a
+// compute unit.
+template <typename E, int D, bool GATHERED>
+__global__ void __launch_bounds__(kWave) stage1_narrow_kernel(Stage1Args a) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int local_vnode = blockIdx.x / a.hkv;
+  narrow_wave<E, D, GATHERED>(a, smem, 0, a.narrow_begin + local_vnode, blockIdx.x - local_vnode * a.hkv);
 }
 
 // Blocks are handed to compute units in index order as units become free, so serving the wide
@@ -1198,13 +1205,23 @@ __global__ void __launch_bounds__(kBlock) stage2_kernel(Stage2Args a) {
     l_run = l_run * keep + group_sum<LPH>(w);
     acc *= keep;
     m_run = m_new;
-#pragma unroll 4
-    for (int i = 0; i < cnt; ++i) {
-      const float wi = __shfl(w, i, LPH);
-      const int ri = __shfl(my_row, i, LPH);
-      if (wi != 0.f) {
-        const f32x4 part = *reinterpret_cast<const f32x4*>(a.mid_o + (int64_t)ri * a.so0 + (int64_t)head * a.so1 + 4 * gl);
-        acc += part * wi;
+    // rows in batches of kBatch: all loads of a batch are issued before the first is used (the
+    // rows are in bounds whatever their weight; a zero weight discards the row's contents)
+    constexpr int kBatch = 8;
+    for (int i0 = 0; i0 < cnt; i0 += kBatch) {
+      f32x4 part[kBatch];
+      float wi[kBatch];
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) {
+        const int i = min(i0 + j, cnt - 1);
+        wi[j] = (i0 + j < cnt) ? __shfl(w, i, LPH) : 0.f;
+        const int ri = __shfl(my_row, i, LPH);
+        part[j] = *reinterpret_cast<const f32x4*>(a.mid_o + (int64_t)ri * a.so0 + (int64_t)head * a.so1 + 4 * gl);
+      }
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] += (wi[j] != 0.f) ? part[j][e] * wi[j] : 0.f;
       }
     }
   }
@@ -1258,6 +1275,16 @@ int launch_stage1_fused(const Stage1Args& a, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? FT_OK : FT_ERR_LAUNCH;
 }
 
+template <typename E, int D, bool GATHERED>
+int launch_stage1_narrow(const Stage1Args& a, hipStream_t stream) {
+  const int64_t blocks = (int64_t)a.narrow_count * a.hkv;
+  if (blocks == 0) return FT_OK;
+  if (blocks > INT32_MAX) return FT_ERR_ARGUMENT;
+  hipLaunchKernelGGL((stage1_narrow_kernel<E, D, GATHERED>), dim3((unsigned)blocks, 1, 1), dim3(kWave, 1, 1),
+                     (size_t)NarrowGeom<D>::kLds, stream, a);
+  return hipGetLastError() == hipSuccess ? FT_OK : FT_ERR_LAUNCH;
+}
+
 // `a` names two vnode ranges: [vnode_begin, +vnode_count) of wide vnodes (more than 16 query
 // rows) and [narrow_begin, +narrow_count) of narrow ones.
 template <typename E, int D, bool GATHERED>
@@ -1274,6 +1301,7 @@ int launch_stage1_d(const Stage1Args& a, hipStream_t stream) {
     }
     return FT_OK;
   } else {
+    if (a.vnode_count == 0) return launch_stage1_narrow<E, D, GATHERED>(a, stream);
     return launch_stage1_fused<E, D, GATHERED>(a, stream);
   }
 }
