@@ -116,7 +116,8 @@ struct Stage1Args {
   const int32_t* q_offs;
   const int32_t* q_lens;
   int vnode_begin, vnode_count;    // vnodes served by 8-wave blocks (or the whole range for the per-wave-staging kernel)
-  int narrow_begin, narrow_count;  // vnodes of at most 16 rows, served by one wave each
+  int narrow_begin, narrow_count;  // vnodes of at most 16 rows
+  int narrow_share;                // waves that share one narrow vnode: 1, 2, 4 or 8
   int g;
   int hkv;
   float scale_log2;  // sm_scale * log2(e)
@@ -939,16 +940,16 @@ template <int D> struct NarrowGeom {
   static __device__ __forceinline__ int swz(int row) { return (((row & 3) << 2) | ((row >> 2) & 3)) & (kChunks - 1); }
 };
 
+// One wave's share of a narrow vnode for the 16 query rows from row0: the tiles tile0,
+// tile0 + tstride, ... of the run, staged in the wave's own LDS area at lds0.
 template <typename E, int D, bool GATHERED>
-__device__ __forceinline__ void narrow_wave(const Stage1Args& a, char* smem, int wave, int vnode, int kvh) {
+__device__ __forceinline__ void narrow_attend(const Stage1Args& a, const VnodeView& vn, char* smem, unsigned lds0,
+                                              int kvh, int row0, int tile0, int tstride, WaveState<D, 1>& st) {
   using N = NarrowGeom<D>;
   constexpr int KS = D / 32, DB = D / 16;
   constexpr float kSlackN = 8.f;
   const int lane = threadIdx.x & 63;
   const int p = lane & 15, c = lane >> 4;
-  const unsigned lds0 = (unsigned)wave * N::kLds;  // the dynamic LDS segment starts at 0
-  const VnodeView vn = load_vnode<GATHERED>(a, vnode);
-  const int rows_total = vn.q_len * a.g;
   const int ntiles = (vn.kv_len + kTileTokens - 1) / kTileTokens;
   int* idx_lds = reinterpret_cast<int*>(smem + lds0 + N::kBytes);
 
@@ -968,126 +969,203 @@ __device__ __forceinline__ void narrow_wave(const Stage1Args& a, char* smem, int
     v_addr[tb] = lds0 + N::kBytesK + vr * N::kRowBytes + 16 * ((((p & 3) >> 1) & (N::kChunks - 1)) ^ N::swz(vr)) + 8 * (p & 1);
   }
 
-  for (int row0 = 0; row0 < rows_total; row0 += 16) {
-    u32x4 qf[1][KS];
-    load_q_frags<D, 1, GATHERED>(a, vn, kvh, row0, qf);
-    WaveState<D, 1> st;
-    reset_state<D, 1>(st);
-    if (ntiles > 0) {
-      int idx_base = 0;
-      auto stage_indices = [&](int base) {
-        if constexpr (!GATHERED) {
-          idx_base = base;
-          // (branch free, so that the loads are in flight together; entries past the run repeat its last)
-          int e[N::kIdxCap / kWave];
+  u32x4 qf[1][KS];
+  load_q_frags<D, 1, GATHERED>(a, vn, kvh, row0, qf);
+  reset_state<D, 1>(st);
+  if (tile0 < ntiles) {
+    // slot indices of tokens [idx_base, idx_base + kIdxCap) of the run
+    int idx_base = 0;
+    auto stage_indices = [&](int base) {
+      if constexpr (!GATHERED) {
+        idx_base = base;
+        // (branch free, so that the loads are in flight together; entries past the run repeat its last)
+        int e[N::kIdxCap / kWave];
 #pragma unroll
-          for (int i = 0; i < N::kIdxCap / kWave; ++i)
-            e[i] = a.kv_entries[vn.kv_base + min(base + kWave * i + lane, vn.kv_len - 1)];
+        for (int i = 0; i < N::kIdxCap / kWave; ++i)
+          e[i] = a.kv_entries[vn.kv_base + min(base + kWave * i + lane, vn.kv_len - 1)];
 #pragma unroll
-          for (int i = 0; i < N::kIdxCap / kWave; ++i) idx_lds[kWave * i + lane] = e[i];
-          wave_lds_fence();
-        }
-      };
-      // K (or V) rows of `tile` -> the wave's K (V) tile.  Tokens past the run repeat its last
-      // token (their scores are masked, their V rows are finite).  The slot indices are read
-      // from the staged window each time rather than kept in registers between the two calls.
-      auto issue = [&](int tile, bool is_v) {
-        if constexpr (!GATHERED) {
-          if (tile * kTileTokens >= idx_base + N::kIdxCap) stage_indices(idx_base + N::kIdxCap);
-        }
+        for (int i = 0; i < N::kIdxCap / kWave; ++i) idx_lds[kWave * i + lane] = e[i];
+        wave_lds_fence();
+      }
+    };
+    // K (or V) rows of `tile` -> the wave's K (V) tile.  Tokens past the run repeat its last
+    // token (their scores are masked, their V rows are finite).  The slot indices are read
+    // from the staged window each time rather than kept in registers between the two calls.
+    auto issue = [&](int tile, bool is_v) {
+      if constexpr (!GATHERED) {
+        if (tile * kTileTokens >= idx_base + N::kIdxCap) stage_indices(tile * kTileTokens);
+      }
 #pragma unroll
-        for (int g = 0; g < N::kGroups; ++g) {
-          const int row = g * N::kGroupRows + grp_row;
-          const int t = min(tile * kTileTokens + row, vn.kv_len - 1);
-          const unsigned srow = GATHERED ? (unsigned)(vn.kv_base + t) : (unsigned)idx_lds[t - idx_base];
-          const char* src = (is_v ? vbase : kbase) + (uint64_t)srow * (is_v ? v_stride : k_stride) + 16 * (pos ^ N::swz(row));
-          load_direct16(src, lds0 + (is_v ? N::kBytesK : 0) + g * 1024);
-        }
-      };
-      stage_indices(0);
-      // nothing the compiler itself tracks may still be in flight below: a wait for it would
-      // also wait for every direct load
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-      issue(0, false);
-      issue(0, true);
-      for (int tile = 0; tile < ntiles; ++tile) {
-        const bool more = tile + 1 < ntiles;
-        const int valid = vn.kv_len - tile * kTileTokens;
-        // ---- S^T = K Q^T : s[tb][j] = score(token 16*tb + 4*c + j, row p)
-        wait_direct_loads<N::kGroups>();  // K landed; V may still be in flight
-        f32x4 s[2];
+      for (int g = 0; g < N::kGroups; ++g) {
+        const int row = g * N::kGroupRows + grp_row;
+        const int t = min(tile * kTileTokens + row, vn.kv_len - 1);
+        const unsigned srow = GATHERED ? (unsigned)(vn.kv_base + t) : (unsigned)idx_lds[t - idx_base];
+        const char* src = (is_v ? vbase : kbase) + (uint64_t)srow * (is_v ? v_stride : k_stride) + 16 * (pos ^ N::swz(row));
+        load_direct16(src, lds0 + (is_v ? N::kBytesK : 0) + g * 1024);
+      }
+    };
+    stage_indices(tile0 * kTileTokens);
+    // nothing the compiler itself tracks may still be in flight below: a wait for it would
+    // also wait for every direct load
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    issue(tile0, false);
+    issue(tile0, true);
+    for (int tile = tile0; tile < ntiles; tile += tstride) {
+      const int next = tile + tstride;
+      const bool more = next < ntiles;
+      const int valid = vn.kv_len - tile * kTileTokens;
+      // ---- S^T = K Q^T : s[tb][j] = score(token 16*tb + 4*c + j, row p)
+      wait_direct_loads<N::kGroups>();  // K landed; V may still be in flight
+      f32x4 s[2];
 #pragma unroll
-        for (int tb = 0; tb < 2; ++tb) {
-          s[tb] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int tb = 0; tb < 2; ++tb) {
+        s[tb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int ks = 0; ks < KS; ++ks) s[tb] = E::mfma(lds_read16(k_addr[tb] ^ (64u * ks)), qf[0][ks], s[tb]);
-          __builtin_amdgcn_sched_barrier(0);  // one token block's operands at a time: keeps the register count low
-        }
-        if (more) {
-          __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the K tile has been read
-          issue(tile + 1, false);
-        }
-        if (valid < kTileTokens) {
-#pragma unroll
-          for (int tb = 0; tb < 2; ++tb)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-              if (16 * tb + 4 * c + j >= valid) s[tb][j] = -INFINITY;
-        }
-        // online soft-max with a lazily updated reference (see tile_step)
-        float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
-                         fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
-        mx = xor32_max(xor16_max(mx)) * a.scale_log2;
-        const bool grow = mx > st.m[0] + kSlackN;
-        if (__builtin_amdgcn_ballot_w64(grow)) {
-          const float m_new = grow ? mx : st.m[0];
-          const float alpha = __builtin_amdgcn_exp2f(st.m[0] - m_new);
-          st.l[0] *= alpha;
-#pragma unroll
-          for (int db = 0; db < DB; ++db) st.o[0][db] *= alpha;
-          st.m[0] = m_new;
-        }
-        const float neg_m = -st.m[0];
-        float x[8];
-        float sum = 0.f;
+        for (int ks = 0; ks < KS; ++ks) s[tb] = E::mfma(lds_read16(k_addr[tb] ^ (64u * ks)), qf[0][ks], s[tb]);
+      }
+      if (more) {
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the K tile has been read
+        issue(next, false);
+      }
+      if (valid < kTileTokens) {
 #pragma unroll
         for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            x[4 * tb + j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tb][j], a.scale_log2, neg_m));
-            sum += x[4 * tb + j];
-          }
-        st.l[0] += sum;
-        const u32x4 pf = {E::pack2(x[0], x[1]), E::pack2(x[2], x[3]), E::pack2(x[4], x[5]), E::pack2(x[6], x[7])};
-        // ---- O^T += V^T P^T
-        if (more) wait_direct_loads<N::kGroups>();  // V landed; the next K may be in flight
-        else wait_direct_loads<0>();
+          for (int j = 0; j < 4; ++j)
+            if (16 * tb + 4 * c + j >= valid) s[tb][j] = -INFINITY;
+      }
+      // online soft-max with a lazily updated reference (see tile_step)
+      float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
+                       fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+      mx = xor32_max(xor16_max(mx)) * a.scale_log2;
+      const bool grow = mx > st.m[0] + kSlackN;
+      if (__builtin_amdgcn_ballot_w64(grow)) {
+        const float m_new = grow ? mx : st.m[0];
+        const float alpha = __builtin_amdgcn_exp2f(st.m[0] - m_new);
+        st.l[0] *= alpha;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const u32x2 lo = lds_read_tr8(v_addr[0] ^ (32u * db));
-          const u32x2 hi = lds_read_tr8(v_addr[1] ^ (32u * db));
-          const u32x4 vf = {lo[0], lo[1], hi[0], hi[1]};
-          st.o[0][db] = E::mfma(vf, pf, st.o[0][db]);
+        for (int db = 0; db < DB; ++db) st.o[0][db] *= alpha;
+        st.m[0] = m_new;
+      }
+      const float neg_m = -st.m[0];
+      float x[8];
+      float sum = 0.f;
+#pragma unroll
+      for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          x[4 * tb + j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[tb][j], a.scale_log2, neg_m));
+          sum += x[4 * tb + j];
         }
-        if (more) {
-          __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the V tile has been read
-          issue(tile + 1, true);
-        }
+      st.l[0] += sum;
+      const u32x4 pf = {E::pack2(x[0], x[1]), E::pack2(x[2], x[3]), E::pack2(x[4], x[5]), E::pack2(x[6], x[7])};
+      // ---- O^T += V^T P^T
+      if (more) wait_direct_loads<N::kGroups>();  // V landed; the next K may be in flight
+      else wait_direct_loads<0>();
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const u32x2 lo = lds_read_tr8(v_addr[0] ^ (32u * db));
+        const u32x2 hi = lds_read_tr8(v_addr[1] ^ (32u * db));
+        const u32x4 vf = {lo[0], lo[1], hi[0], hi[1]};
+        st.o[0][db] = E::mfma(vf, pf, st.o[0][db]);
+      }
+      if (more) {
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the V tile has been read
+        issue(next, true);
       }
     }
-    finish_state<D, 1>(st);
-    write_partials<D, 1>(a, vn, kvh, row0, st);
+  }
+  finish_state<D, 1>(st);
+}
+
+// Merge of the `share` waves of one narrow vnode (same rows, interleaved tiles) into the first of
+// them, pairwise through LDS at xchg.  Every wave of the block calls this (block barriers).
+template <int D>
+__device__ __forceinline__ void merge_shares(float* xchg, WaveState<D, 1>& st, int w, int share) {
+  constexpr int NV = (D / 16) * 4 + 2;  // floats of state per lane
+  const int lane = threadIdx.x & 63;
+  for (int half = share >> 1; half >= 1; half >>= 1) {
+    __syncthreads();
+    if (w >= half && w < 2 * half) {
+      float* dst = xchg + (size_t)(w - half) * NV * kWave + lane;
+      int n = 0;
+      dst[(n++) * kWave] = st.m[0];
+      dst[(n++) * kWave] = st.l[0];
+#pragma unroll
+      for (int db = 0; db < D / 16; ++db)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dst[(n++) * kWave] = st.o[0][db][j];
+    }
+    __syncthreads();
+    if (w < half) {
+      const float* src = xchg + (size_t)w * NV * kWave + lane;
+      int n = 0;
+      const float m2 = src[(n++) * kWave];
+      const float l2 = src[(n++) * kWave];
+      const float m = fmaxf(st.m[0], m2);
+      const float a1 = scale_from(st.m[0], m), a2 = scale_from(m2, m);
+      st.l[0] = st.l[0] * a1 + l2 * a2;
+      st.m[0] = m;
+#pragma unroll
+      for (int db = 0; db < D / 16; ++db)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) st.o[0][db][j] = st.o[0][db][j] * a1 + src[(n++) * kWave] * a2;
+    }
   }
 }
 
-// Narrow vnodes alone (a launch without wide vnodes), one wave per block: the footprint of one
-// LDS tile instead of a wide block's ring, so that more of these latency-bound waves share a
-// compute unit.
+// A narrow vnode served by `share` consecutive waves of a block (share = 1, 2, 4 or 8, the same
+// for the whole launch; the host picks more than one when there are fewer vnodes than wave
+// slots): wave w of the vnode takes the tiles w, w + share, ..., and the shares are merged
+// through LDS.  `slot` is the wave's index in the block; a wave without a vnode (exists ==
+// false) only keeps the block's barriers company.
 template <typename E, int D, bool GATHERED>
-__global__ void __launch_bounds__(kWave) stage1_narrow_kernel(Stage1Args a) {
+__device__ __forceinline__ void narrow_item(const Stage1Args& a, char* smem, int slot, int share, bool exists,
+                                            int vnode, int kvh) {
+  using N = NarrowGeom<D>;
+  const unsigned lds0 = (unsigned)slot * N::kLds;  // the dynamic LDS segment starts at 0
+  VnodeView vn{0, 0, 0, 0};
+  if (exists) vn = load_vnode<GATHERED>(a, vnode);
+  const int rows_total = vn.q_len * a.g;
+  if (share == 1) {
+    for (int row0 = 0; row0 < rows_total; row0 += 16) {
+      WaveState<D, 1> st;
+      narrow_attend<E, D, GATHERED>(a, vn, smem, lds0, kvh, row0, 0, 1, st);
+      write_partials<D, 1>(a, vn, kvh, row0, st);
+    }
+    return;
+  }
+  const int w = slot & (share - 1);
+  float* xchg = reinterpret_cast<float*>(smem + (size_t)(slot - w) * N::kLds);
+  // every wave of the block makes the same number of passes (block barriers inside): the most
+  // any of its vnodes needs, agreed on through one word of each wave's LDS area
+  const int nwaves = blockDim.x >> 6;
+  *reinterpret_cast<volatile int*>(smem + lds0) = (rows_total + 15) >> 4;
+  __syncthreads();
+  int passes = 0;
+  for (int i = 0; i < nwaves; ++i) passes = max(passes, *reinterpret_cast<volatile int*>(smem + (size_t)i * N::kLds));
+  __syncthreads();
+  for (int pass = 0; pass < passes; ++pass) {
+    const int row0 = 16 * pass;
+    WaveState<D, 1> st;
+    if (row0 < rows_total) narrow_attend<E, D, GATHERED>(a, vn, smem, lds0, kvh, row0, w, share, st);
+    else reset_state<D, 1>(st);
+    merge_shares<D>(xchg, st, w, share);
+    if (w == 0 && row0 < rows_total) write_partials<D, 1>(a, vn, kvh, row0, st);
+    __syncthreads();  // the exchange area is the staging area of the next pass
+  }
+}
+
+// Narrow vnodes alone (a launch without wide vnodes), one vnode per block of `narrow_share`
+// waves: the footprint of one LDS tile per wave instead of a wide block's ring, so that more of
+// these latency-bound waves share a compute unit.
+template <typename E, int D, bool GATHERED>
+__global__ void __launch_bounds__(kWideBlock) stage1_narrow_kernel(Stage1Args a) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int local_vnode = blockIdx.x / a.hkv;
-  narrow_wave<E, D, GATHERED>(a, smem, 0, a.narrow_begin + local_vnode, blockIdx.x - local_vnode * a.hkv);
+  narrow_item<E, D, GATHERED>(a, smem, wave, a.narrow_share, true, a.narrow_begin + local_vnode,
+                              blockIdx.x - local_vnode * a.hkv);
 }
 
 // Blocks are handed to compute units in index order as units become free, so serving the wide
@@ -1133,12 +1211,14 @@ __global__ void __launch_bounds__(kWideBlock) stage1_fused_kernel(Stage1Args a) 
     wide_block<E, D, GATHERED>(a, smem, local_vnode, blockIdx.x - rank * a.hkv);
   } else {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int item = (blockIdx.x - wide_blocks) * kWideWaves + wave;
-    if (item >= a.narrow_count * a.hkv) return;  // whole wave; no block barrier below
+    const int share = a.narrow_share;
+    const int item = (blockIdx.x - wide_blocks) * (kWideWaves / share) + wave / share;
+    const bool exists = item < a.narrow_count * a.hkv;
+    if (share == 1 && !exists) return;  // whole wave; no block barrier below in this mode
     const int local_vnode = item / a.hkv;
     const int kvh = item - local_vnode * a.hkv;
     FT_TIME(unsigned long long t_start = FT_CLOCK(); unsigned long long rt_start = wall_clock64();)
-    narrow_wave<E, D, GATHERED>(a, smem, wave, a.narrow_begin + local_vnode, kvh);
+    narrow_item<E, D, GATHERED>(a, smem, wave, share, exists, a.narrow_begin + local_vnode, kvh);
     FT_TIME(if (g_timing && (threadIdx.x & 63) == 0) {
       unsigned long long* out = g_timing + ((size_t)blockIdx.x * kWideWaves + wave) * 8;
       out[4] = FT_CLOCK() - t_start; out[5] = 0; out[6] = rt_start; out[7] = wall_clock64();
@@ -1253,8 +1333,27 @@ int launch_stage1_inst(const Stage1Args& a, int hkv, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? FT_OK : FT_ERR_LAUNCH;
 }
 
+// Waves that share one narrow vnode: the largest power of two (at most 8) that fills at most
+// three quarters of the wave slots (8 per compute unit).  With far fewer vnodes than slots the
+// waves would each walk a long run alone, one memory round trip per tile; with the slots nearly
+// full the runs are limited by memory bandwidth already and sharing only adds barriers.
+inline int narrow_share_for(int64_t items) {
+  static int slots = 0;
+  if (slots == 0) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+      (void)hipGetLastError();
+      cus = 256;
+    }
+    slots = cus * kWideWaves;
+  }
+  int share = 1;
+  while (share < kWideWaves && 4 * items * (2 * share) <= 3 * (int64_t)slots) share *= 2;
+  return share;
+}
+
 template <typename E, int D, bool GATHERED>
-int launch_stage1_fused(const Stage1Args& a, hipStream_t stream) {
+int launch_stage1_fused(const Stage1Args& a0, hipStream_t stream) {
   constexpr size_t kWideLds = (size_t)WideGeom<D>::kLds;
   constexpr size_t kNarrowLds = (size_t)kWideWaves * NarrowGeom<D>::kLds;
   constexpr size_t lds = kWideLds > kNarrowLds ? kWideLds : kNarrowLds;
@@ -1267,8 +1366,11 @@ int launch_stage1_fused(const Stage1Args& a, hipStream_t stream) {
     }
     configured = true;
   }
+  Stage1Args a = a0;
   const int64_t narrow_items = (int64_t)a.narrow_count * a.hkv;
-  const int64_t blocks = (int64_t)a.vnode_count * a.hkv + (narrow_items + kWideWaves - 1) / kWideWaves;
+  a.narrow_share = narrow_share_for(narrow_items);
+  const int per_block = kWideWaves / a.narrow_share;
+  const int64_t blocks = (int64_t)a.vnode_count * a.hkv + (narrow_items + per_block - 1) / per_block;
   if (blocks == 0) return FT_OK;
   if (blocks > INT32_MAX) return FT_ERR_ARGUMENT;
   hipLaunchKernelGGL(kern, dim3((unsigned)blocks, 1, 1), dim3(kWideBlock, 1, 1), lds, stream, a);
@@ -1276,12 +1378,24 @@ int launch_stage1_fused(const Stage1Args& a, hipStream_t stream) {
 }
 
 template <typename E, int D, bool GATHERED>
-int launch_stage1_narrow(const Stage1Args& a, hipStream_t stream) {
+int launch_stage1_narrow(const Stage1Args& a0, hipStream_t stream) {
+  Stage1Args a = a0;
   const int64_t blocks = (int64_t)a.narrow_count * a.hkv;
   if (blocks == 0) return FT_OK;
   if (blocks > INT32_MAX) return FT_ERR_ARGUMENT;
-  hipLaunchKernelGGL((stage1_narrow_kernel<E, D, GATHERED>), dim3((unsigned)blocks, 1, 1), dim3(kWave, 1, 1),
-                     (size_t)NarrowGeom<D>::kLds, stream, a);
+  a.narrow_share = narrow_share_for(blocks);
+  auto kern = stage1_narrow_kernel<E, D, GATHERED>;
+  const size_t lds = (size_t)a.narrow_share * NarrowGeom<D>::kLds;
+  static bool configured = false;  // raising the dynamic LDS limit is idempotent
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kWideWaves * NarrowGeom<D>::kLds) != hipSuccess) {
+      (void)hipGetLastError();
+      return FT_ERR_LAUNCH;
+    }
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks, 1, 1), dim3(kWave * a.narrow_share, 1, 1), lds, stream, a);
   return hipGetLastError() == hipSuccess ? FT_OK : FT_ERR_LAUNCH;
 }
 
