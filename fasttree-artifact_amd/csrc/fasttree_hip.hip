@@ -685,6 +685,18 @@ __device__ __forceinline__ void tile_step32(const WideLane& la, unsigned off, in
   }
 
   FT_TIME(__builtin_amdgcn_sched_barrier(0); const unsigned long long tc1 = FT_CLOCK(); __builtin_amdgcn_sched_barrier(0);)
+  // the V^T operands do not depend on the probabilities: request them now, so that they arrive
+  // under the soft-max arithmetic (they take the registers the K operands just left)
+  const unsigned vlo = la.v_lo + off, vhi = la.v_hi + off;
+  u32x4 vf[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int u = i / DB, db = i % DB;
+    const u32x2 lo = lds_read_tr8((vlo ^ (64u * db)) + u * 16 * W::kRowBytes);
+    const u32x2 hi = lds_read_tr8((vhi ^ (64u * db)) + u * 16 * W::kRowBytes);
+    vf[i] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+  }
+  __builtin_amdgcn_sched_barrier(0);
   float mx = max3(s[0], s[1], s[2]);
 #pragma unroll
   for (int j = 3; j < 15; j += 2) mx = max3(mx, s[j], s[j + 1]);
@@ -715,15 +727,8 @@ __device__ __forceinline__ void tile_step32(const WideLane& la, unsigned off, in
                   E::pack2(x[8 * u + 4], x[8 * u + 5]), E::pack2(x[8 * u + 6], x[8 * u + 7])};
 
   FT_TIME(__builtin_amdgcn_sched_barrier(0); const unsigned long long tc2 = FT_CLOCK(); __builtin_amdgcn_sched_barrier(0);)
-  const unsigned vlo = la.v_lo + off, vhi = la.v_hi + off;
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int u = i / DB, db = i % DB;
-    const u32x2 lo = lds_read_tr8((vlo ^ (64u * db)) + u * 16 * W::kRowBytes);
-    const u32x2 hi = lds_read_tr8((vhi ^ (64u * db)) + u * 16 * W::kRowBytes);
-    const u32x4 vf = {lo[0], lo[1], hi[0], hi[1]};
-    st.o[db] = E::mfma32(vf, pf[u], st.o[db]);
-  }
+  for (int i = 0; i < NV; ++i) st.o[i % DB] = E::mfma32(vf[i], pf[i / DB], st.o[i % DB]);
   FT_TIME(if (tt) { __builtin_amdgcn_sched_barrier(0); const unsigned long long tc3 = FT_CLOCK(); tt[0] += tc1 - tc0; tt[1] += tc2 - tc1; tt[2] += tc3 - tc2; tt[3] += 1; })
 }
 
