@@ -16,6 +16,7 @@
 // (stage 2), :582-642 (the call that chains them).
 
 #include <hip/hip_runtime.h>
+#include <algorithm>
 #include <stdint.h>
 
 #include "../../include/fasttree_hip.h"
@@ -115,9 +116,11 @@ struct Stage1Args {
   const int32_t* q_entries;
   const int32_t* q_offs;
   const int32_t* q_lens;
-  int vnode_begin, vnode_count;    // vnodes served by 8-wave blocks (or the whole range for the per-wave-staging kernel)
+  int vnode_begin, vnode_count;    // vnodes served by wide blocks (or the whole range for the per-wave-staging kernel)
   int narrow_begin, narrow_count;  // vnodes of at most 16 rows
   int narrow_share;                // waves that share one narrow vnode: 1, 2, 4 or 8
+  int wide_rows;                   // query rows the planner's tile gives a wide vnode (host hint for wide_chunks)
+  int wide_chunks;                 // blocks per (wide vnode, kv head); block c serves row pieces c, c + wide_chunks, ..
   int g;
   int hkv;
   float scale_log2;  // sm_scale * log2(e)
@@ -507,9 +510,10 @@ __global__ void __launch_bounds__(kBlock) stage1_kernel(Stage1Args a) {
 }
 
 // ---------------------------------------------------------------------------------------
-// Wide vnodes: 32x32x16 MFMA tiles (twice the rate of 16x16x32 on this part), 8 waves per
-// block with 32 query rows each, so that two waves share a SIMD and one wave's soft-max
-// arithmetic overlaps the other's matrix instructions.
+// Wide vnodes: 32x32x16 MFMA tiles (twice the rate of 16x16x32 on this part), four waves per
+// block with 32 query rows each and two blocks per compute unit, so that two waves share a SIMD
+// and one wave's waits are filled by the other's instructions.  (Matrix and vector arithmetic
+// of the two do not run at the same time on this part: a tile step costs the sum of both.)
 // ---------------------------------------------------------------------------------------
 #ifdef FT_TIMING
 // Development aid, compiled out of the product: per-wave cycle counts of the wide kernel's
@@ -521,17 +525,22 @@ __device__ int g_timing_steps = 0;  // 1: report per-step phases (scores, soft-m
 #else
 #define FT_TIME(...)
 #endif
-constexpr int kWideWaves = 8;
-constexpr int kWideBlock = kWave * kWideWaves;
+#ifndef FT_WIDE_WAVES
+#define FT_WIDE_WAVES 4
+#endif
 #ifndef FT_WIDE_BUFS
-#define FT_WIDE_BUFS 4
+#define FT_WIDE_BUFS 2
 #endif
 #ifndef FT_WIDE_IDX
-#define FT_WIDE_IDX 4096
+#define FT_WIDE_IDX 2048
 #endif
+constexpr int kWideWaves = FT_WIDE_WAVES;
+constexpr int kWideBlock = kWave * kWideWaves;
+constexpr int kWideRows = 32 * kWideWaves;        // query rows one pass of a block serves
+constexpr int kWaveSlotsPerCu = 8;                // waves of these kernels a compute unit holds
 
 // LDS layout of the wide kernel: rows of 2*D bytes back to back (no padding), 64-token super
-// tiles of two 32-token tiles, a ring of four buffers, then a staging area for the run's slot
+// tiles of two 32-token tiles, a ring of kBufs buffers, then a staging area for the run's slot
 // indices.  A row's 16-byte chunks are stored XOR-permuted: chunk c of row r sits in slot
 // c ^ swz(r).  swz swaps the two low bit pairs of r, which makes both read patterns conflict free
 // for 256-byte rows: the K operand read (16 different rows, same chunk) and the transposed V
@@ -795,15 +804,15 @@ __device__ __forceinline__ void merge_token_groups(float* xchg, WideState<D>& st
   }
 }
 
-// One block (8 waves) per (vnode, kv head).  The block streams the vnode's KV run through a ring
-// of four 64-token LDS buffers with direct global->LDS loads, three super tiles ahead of the one
-// being consumed; the run's slot indices are staged in LDS first so that nothing but those
-// loads is in flight in the loop.  Per pass over the run the waves form RG row groups of 32
-// query rows x TG token groups (RG * TG = 8, or 4 when only 32 rows are left): a wave consumes
-// the 32-token tiles t with t % TG == tg for the rows of its row group, and the TG states of a
-// row group are merged at the end.
+// One block (kWideWaves waves) per (vnode, kv head, chunk of kWideRows query rows).  The block
+// streams the vnode's KV run through a ring of kBufs 64-token LDS buffers with direct
+// global->LDS loads, kBufs - 1 super tiles ahead of the one being consumed; the run's slot
+// indices are staged in LDS first so that nothing but those loads is in flight in the loop.
+// Per pass over the run the waves form RG row groups of 32 query rows x TG token groups
+// (RG * TG = kWideWaves): a wave consumes the 32-token tiles t with t % TG == tg for the rows of
+// its row group, and the TG states of a row group are merged at the end.
 template <typename E, int D, bool GATHERED>
-__device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int local_vnode, int kvh) {
+__device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int local_vnode, int kvh, int chunk) {
   using W = WideGeom<D>;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const VnodeView vn = load_vnode<GATHERED>(a, a.vnode_begin + local_vnode);
@@ -817,13 +826,21 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
   const unsigned k_stride = (unsigned)(2 * a.sk0), v_stride = (unsigned)(2 * a.sv0);  // bytes, < 2^32 (checked by the host)
   int* idx_lds = reinterpret_cast<int*>(smem + W::kRing);
 
-  for (int row0 = 0; row0 < rows_total;) {
-    const int groups = (rows_total - row0 + 31) >> 5;   // 32-row groups still to serve
-    const int tgroups = groups >= 5 ? 1 : (groups >= 3 ? 2 : 4);
-    const int rgroups = groups >= 5 ? 8 : (groups >= 3 ? 4 : (groups == 2 ? 2 : 1));
+  // this block's pieces of kWideRows rows: chunk, chunk + wide_chunks, ...
+  for (int piece = chunk; piece * kWideRows < rows_total; piece += a.wide_chunks) {
+  const int rows_end = min((piece + 1) * kWideRows, rows_total);
+  for (int row0 = piece * kWideRows; row0 < rows_end;) {
+    // waves as rgroups row groups x tgroups token groups: halve the row groups (down to a token
+    // split of four) while the rows left in the piece leave half of them without rows
+    const int groups = (rows_end - row0 + 31) >> 5;   // 32-row groups still to serve
+    int rgroups = kWideWaves, tgroups = 1;
+    while (tgroups < 4 && 2 * groups <= rgroups) {
+      rgroups >>= 1;
+      tgroups <<= 1;
+    }
     const int rg = wave / tgroups, tg = wave % tgroups;
     const int my_row0 = row0 + 32 * rg;
-    const bool active = rg < rgroups && my_row0 < rows_total;
+    const bool active = rg < rgroups && my_row0 < rows_end;
 
     u32x4 qf[D / 16];
     load_q_frags32<D, GATHERED>(a, vn, kvh, active ? my_row0 : rows_total, qf);
@@ -922,6 +939,7 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
     if (active && tg == 0) write_partials32<D>(a, vn, kvh, my_row0, st);
     __syncthreads();  // staging LDS is reused by the next pass over the run
     row0 += 32 * rgroups;
+  }
   }
 }
 
@@ -1206,18 +1224,26 @@ __device__ __forceinline__ int wide_vnode_of_rank(const Stage1Args& a, char* sme
   return v;
 }
 
+// Launch order of the fused kernel.  Wide blocks come rank-major, then row chunk, kv head fastest
+// (blocks that stream the same KV run are launched together and share it in L2); the narrow
+// blocks follow and fill the machine while the wide blocks drain.
 template <typename E, int D, bool GATHERED>
-__global__ void __launch_bounds__(kWideBlock) stage1_fused_kernel(Stage1Args a) {
+__global__ void __launch_bounds__(kWideBlock, 512 / kWideBlock) stage1_fused_kernel(Stage1Args a) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  const int wide_blocks = a.vnode_count * a.hkv;
-  if ((int)blockIdx.x < wide_blocks) {
-    const int rank = blockIdx.x / a.hkv;
+  const int wide_blocks = a.vnode_count * a.wide_chunks * a.hkv;
+  const int wide_index = blockIdx.x, narrow_index = (int)blockIdx.x - wide_blocks;
+  const bool is_wide = (int)blockIdx.x < wide_blocks;
+  if (is_wide) {
+    const int per_rank = a.wide_chunks * a.hkv;
+    const int rank = wide_index / per_rank;
+    const int rest = wide_index - rank * per_rank;
+    const int chunk = rest / a.hkv;
     const int local_vnode = wide_vnode_of_rank<GATHERED>(a, smem, rank);
-    wide_block<E, D, GATHERED>(a, smem, local_vnode, blockIdx.x - rank * a.hkv);
+    wide_block<E, D, GATHERED>(a, smem, local_vnode, rest - chunk * a.hkv, chunk);
   } else {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int share = a.narrow_share;
-    const int item = (blockIdx.x - wide_blocks) * (kWideWaves / share) + wave / share;
+    const int item = narrow_index * (kWideWaves / share) + wave / share;
     const bool exists = item < a.narrow_count * a.hkv;
     if (share == 1 && !exists) return;  // whole wave; no block barrier below in this mode
     const int local_vnode = item / a.hkv;
@@ -1350,7 +1376,7 @@ inline int narrow_share_for(int64_t items) {
       (void)hipGetLastError();
       cus = 256;
     }
-    slots = cus * kWideWaves;
+    slots = cus * kWaveSlotsPerCu;
   }
   int share = 1;
   while (share < kWideWaves && 4 * items * (2 * share) <= 3 * (int64_t)slots) share *= 2;
@@ -1375,7 +1401,9 @@ int launch_stage1_fused(const Stage1Args& a0, hipStream_t stream) {
   const int64_t narrow_items = (int64_t)a.narrow_count * a.hkv;
   a.narrow_share = narrow_share_for(narrow_items);
   const int per_block = kWideWaves / a.narrow_share;
-  const int64_t blocks = (int64_t)a.vnode_count * a.hkv + (narrow_items + per_block - 1) / per_block;
+  const int64_t narrow_blocks = (narrow_items + per_block - 1) / per_block;
+  a.wide_chunks = std::max(1, std::min(8, (a.wide_rows + kWideRows - 1) / kWideRows));
+  const int64_t blocks = (int64_t)a.vnode_count * a.wide_chunks * a.hkv + narrow_blocks;
   if (blocks == 0) return FT_OK;
   if (blocks > INT32_MAX) return FT_ERR_ARGUMENT;
   hipLaunchKernelGGL(kern, dim3((unsigned)blocks, 1, 1), dim3(kWideBlock, 1, 1), lds, stream, a);
@@ -1562,6 +1590,7 @@ int ft_stage1(const void* q, const void* k, const void* v,
     a.narrow_begin = vnode_begin; a.narrow_count = vnode_count;
   } else {
     a.vnode_begin = vnode_begin; a.vnode_count = vnode_count;
+    a.wide_rows = (int)std::min<int64_t>((int64_t)q_tile * kv_group_num, 1 << 20);
   }
   return launch_stage1<false>(a, head_dim, dtype, stream);
 }
@@ -1615,6 +1644,8 @@ int ft_stage1_phases(const void* q, const void* k, const void* v,
     if (is_narrow_range) { t.narrow_begin = begin; t.narrow_count = count; }
     else { t.vnode_begin = begin; t.vnode_count = count; }
   };
+  const int64_t widest_tile = std::max(narrow[0] ? 0 : phase_q_tile_sizes[0], narrow[1] ? 0 : phase_q_tile_sizes[1]);
+  a.wide_rows = (int)std::min<int64_t>(widest_tile * g, 1 << 20);
   // Both phases go into one launch when one is wide and the other narrow, or when they are of
   // the same kind and adjacent in the vnode list (the planner's lists always are).
   if (pending[0] && pending[1] && narrow[0] == narrow[1]) {
@@ -1682,7 +1713,7 @@ int ft_gathered_decode(const void* q, const void* k_cache, const void* v_cache,
   a.sk0 = a.sv0 = (int64_t)num_kv_heads * head_dim;
   a.sk1 = a.sv1 = head_dim;
   if (is_narrow(1, g)) { a.narrow_begin = 0; a.narrow_count = batch_size * nsplit; }
-  else { a.vnode_begin = 0; a.vnode_count = batch_size * nsplit; }
+  else { a.vnode_begin = 0; a.vnode_count = batch_size * nsplit; a.wide_rows = g; }
   a.g = g;
   a.hkv = num_kv_heads;
   a.scale_log2 = sm_scale * kLog2e;
