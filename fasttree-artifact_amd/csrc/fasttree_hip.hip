@@ -1018,12 +1018,18 @@ __device__ __forceinline__ void narrow_attend(const Stage1Args& a, const VnodeVi
       if constexpr (!GATHERED) {
         if (tile * kTileTokens >= idx_base + N::kIdxCap) stage_indices(tile * kTileTokens);
       }
+      // (all index reads first: a load instruction is a fence for the compiler, so reads placed
+      // between the loads would each be waited for on its own)
+      unsigned srow[N::kGroups];
+#pragma unroll
+      for (int g = 0; g < N::kGroups; ++g) {
+        const int t = min(tile * kTileTokens + g * N::kGroupRows + grp_row, vn.kv_len - 1);
+        srow[g] = GATHERED ? (unsigned)(vn.kv_base + t) : (unsigned)idx_lds[t - idx_base];
+      }
 #pragma unroll
       for (int g = 0; g < N::kGroups; ++g) {
         const int row = g * N::kGroupRows + grp_row;
-        const int t = min(tile * kTileTokens + row, vn.kv_len - 1);
-        const unsigned srow = GATHERED ? (unsigned)(vn.kv_base + t) : (unsigned)idx_lds[t - idx_base];
-        const char* src = (is_v ? vbase : kbase) + (uint64_t)srow * (is_v ? v_stride : k_stride) + 16 * (pos ^ N::swz(row));
+        const char* src = (is_v ? vbase : kbase) + (uint64_t)srow[g] * (is_v ? v_stride : k_stride) + 16 * (pos ^ N::swz(row));
         load_direct16(src, lds0 + (is_v ? N::kBytesK : 0) + g * 1024);
       }
     };
