@@ -50,6 +50,11 @@ WORKLOADS = {
 # (kernel_bench/benchmark.py:246-254, run_benchmark.sh:46-53: query tiles (64 // g, 16 // g)).
 # "mi355x" = the same planner with a wide-phase query tile of 256 // g requests (256 query
 # rows, the eight waves of a block) and thresholds sized for 256 compute units.
+# HBM bytes per stage-1 launch (read + write) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
+# each scaled by what the same counter reads for a plain copy of known size (2.000 and 1.000); the
+# runs and their commands are summarised in profiles/stage1_fused_stage2_<workload>_<dtype>.txt.
+MEASURED_TRAFFIC = {("c3", "mi355x", "stage1"): 148.9e6, ("c4", "mi355x", "stage1"): 8713.8e6}
+
 PRESETS = {
     "reference": dict(q_tiles=None, kv_tiles=(32, 32), kv_splits=(1024, 128), thr1=(132, 528), thr2=(132, 132)),
     "mi355x": dict(q_tiles="wide", kv_tiles=(32, 32), kv_splits=(1024, 128), thr1=(256, 1024), thr2=(256, 256)),
@@ -228,15 +233,16 @@ def main():
     }
     dom_us = per_launch[dominant]
     dom = work[dominant]
+    traffic = MEASURED_TRAFFIC.get((args.workload, args.preset, dominant))
     mfma_frac = dom["flops"] / (dom_us * 1e-6) / 1e12 / MFMA_PEAK_TFLOPS
     hbm_frac = dom["bytes"] / (dom_us * 1e-6) / 1e9 / HBM_PEAK_GBS
     if mfma_frac >= hbm_frac:
         roofline = {"kernel": dominant, "bound": "mfma", "achieved": dom["flops"] / (dom_us * 1e-6) / 1e12,
-                    "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": mfma_frac, "traffic": None,
+                    "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": mfma_frac, "traffic": traffic,
                     "avg_launch_us": dom_us}
     else:
         roofline = {"kernel": dominant, "bound": "hbm", "achieved": dom["bytes"] / (dom_us * 1e-6) / 1e9,
-                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": hbm_frac, "traffic": None, "avg_launch_us": dom_us}
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": hbm_frac, "traffic": traffic, "avg_launch_us": dom_us}
 
     # ---- the no-sharing baseline on the GPU: per-request gathered cache through the same kernels
     gathered = None
