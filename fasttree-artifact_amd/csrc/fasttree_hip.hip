@@ -900,6 +900,9 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
     // nothing the compiler itself tracks (the Q fragments) may still be in flight in the loop:
     // a wait for it there would also wait for every direct load
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    // (and the compiler must see the fragments as complete, or it keeps a wait for them in the loop)
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(qf[ks]));
 #pragma unroll
     for (int j = 0; j < W::kAhead; ++j) issue_rows(j);
     FT_TIME(unsigned long long t_start = FT_CLOCK(); unsigned long long rt_start = wall_clock64(); unsigned long long t_wait = 0, t_bar = 0, t_issue = 0, t_comp = 0; unsigned long long t_step[4] = {0, 0, 0, 0};)
@@ -1037,6 +1040,9 @@ __device__ __forceinline__ void narrow_attend(const Stage1Args& a, const VnodeVi
     // nothing the compiler itself tracks may still be in flight below: a wait for it would
     // also wait for every direct load
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    // (and the compiler must see the fragments as complete, or it keeps a wait for them in the loop)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[0][ks]));
     issue(tile0, false);
     issue(tile0, true);
     for (int tile = tile0; tile < ntiles; tile += tstride) {
