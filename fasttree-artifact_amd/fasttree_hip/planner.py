@@ -19,15 +19,23 @@ Reference: kernel_bench/fasttree.py:7-27 (parameters), :30-61 (cost model),
 
 from __future__ import annotations
 
+import os
 from collections import deque
 from dataclasses import dataclass, field
 from typing import List, Optional, Sequence, Tuple
 
 import numpy as np
 
+from . import _plan_lib
+
 #: The reference prints its parallelism estimates, final tile/split sizes and the
 #: per-phase vnode counts on every call.  Set to False to silence the planner.
 VERBOSE = True
+
+#: Which implementation ``fasttree_plan`` runs: "native" (libfasttree_plan.so, the C++ planner
+#: behind include/fasttree_plan.h), "python" (this module), or "auto": native when the library is
+#: built and the arguments fit its 32-bit interface.  Both produce identical plans.
+BACKEND = os.environ.get("FASTTREE_PLANNER", "auto")
 
 #: Number of -1 entries appended to the two entry arrays (kernel_bench/fasttree.py:261-262).
 ENTRY_PADDING = 32
@@ -228,6 +236,56 @@ def _estimate_parallelism(tree_info, assignment, served, q_tiles, kv_splits, num
     return [b * num_kv_heads for b in blocks]
 
 
+def _fits_native(KV_ptrs, KV_SPLIT_SIZES, para_threshs1, para_threshs2, params) -> bool:
+    """The native planner takes tile sizes, split sizes, thresholds and token positions as int32."""
+    limit = 2 ** 31 - 1 - ENTRY_PADDING
+    small = [*KV_SPLIT_SIZES[:2], *para_threshs1[:2], *para_threshs2[:2], *params.TSQs[:2], *params.TSKs[:2],
+             params.kv_group_num]
+    return (all(isinstance(x, (int, np.integer)) and 1 <= x <= limit for x in small[:2] + small[6:])
+            and all(isinstance(x, (int, np.integer)) and -limit <= x <= limit for x in small[2:6])
+            and len(KV_ptrs) > 0 and int(KV_ptrs[-1]) <= limit)
+
+
+def _plan_native(tree_info, KV_ptrs, batch_size, num_kv_heads, KV_SPLIT_SIZES, para_threshs1, para_threshs2,
+                 params: FastTreeParams, kv_slot_map) -> FastTreePlan:
+    """``fasttree_plan`` through libfasttree_plan.so: same result, same printed lines, same
+    replacement of ``params.TSQs`` / ``params.TSKs`` when the second adaptation pass fires."""
+    L = _plan_lib
+    r = L.plan(tree_info, KV_ptrs, batch_size, num_kv_heads, KV_SPLIT_SIZES, para_threshs1, para_threshs2,
+               params.alpha, params.beta, params.gamma, params.TSQs, params.TSKs, params.kv_group_num,
+               kv_slot_map=kv_slot_map)
+    history = r[L.PARALLELISMS].reshape(-1, 2).tolist()
+    for para in history:
+        _say("parallelisms:", para)
+    q_tiles = r[L.Q_TILE_SIZES].tolist()
+    if int(r[L.TILES_REPLACED][0]):
+        params.set_q_tile_sizes(q_tiles)
+        params.set_kv_tile_sizes(r[L.KV_TILE_SIZES].tolist())
+    kv_splits = r[L.KV_SPLIT_SIZES].tolist()
+    _say(q_tiles)
+    _say(kv_splits)
+    nums = r[L.PHASE_NODE_NUMS].tolist()
+    _say("Above threshold: ", nums[0])
+    _say("Below threshold: ", nums[1])
+    return FastTreePlan(
+        vnode_to_kv_entries=r[L.KV_ENTRIES],
+        vnode_to_kv_offs=r[L.KV_OFFS].tolist(),
+        vnode_to_kv_lens=r[L.KV_LENS].tolist(),
+        vnode_to_q_entries=r[L.Q_ENTRIES].tolist(),
+        vnode_to_q_offs=r[L.Q_OFFS].tolist(),
+        vnode_to_q_lens=r[L.Q_LENS].tolist(),
+        req_to_vnode_entries=r[L.REQ_ENTRIES].tolist(),
+        req_to_vnode_offs=r[L.REQ_OFFS].tolist(),
+        req_to_vnode_lens=r[L.REQ_LENS].tolist(),
+        phase_node_nums=nums,
+        phase_node_offsets=r[L.PHASE_NODE_OFFSETS].tolist(),
+        node_assignments=r[L.NODE_ASSIGNMENTS].tolist(),
+        q_tile_sizes=list(q_tiles),
+        kv_split_sizes=kv_splits,
+        parallelisms=history,
+    )
+
+
 def fasttree_plan(
     tree_info,
     KV_ptrs: Sequence[int],
@@ -238,14 +296,23 @@ def fasttree_plan(
     para_threshs2: Sequence[int],
     params: FastTreeParams,
     kv_slot_map: Optional[np.ndarray] = None,
+    backend: Optional[str] = None,
 ) -> FastTreePlan:
     """Run the planner and return host-side lists (kernel_bench/fasttree.py:111-262).
+
+    ``backend`` overrides the module's ``BACKEND`` for this call.
 
     ``kv_slot_map`` (optional, length ``KV_ptrs[-1]``) maps the logical token position
     ``KV_ptrs[node] + t`` to the slot of the KV pool that holds it; without it the pool
     is node-major and the entries are the logical positions themselves, as in the
     reference's bench.
     """
+    choice = backend or BACKEND
+    if choice == "native" or (choice == "auto" and _plan_lib.available() and _fits_native(
+            KV_ptrs, KV_SPLIT_SIZES, para_threshs1, para_threshs2, params)):
+        return _plan_native(tree_info, KV_ptrs, batch_size, num_kv_heads, KV_SPLIT_SIZES, para_threshs1,
+                            para_threshs2, params, kv_slot_map)
+
     count = len(tree_info)
     q_tiles = params.TSQs                       # alias on purpose, as in the reference
     kv_splits = [KV_SPLIT_SIZES[0], KV_SPLIT_SIZES[0]]

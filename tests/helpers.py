@@ -40,14 +40,14 @@ def params_for(case) -> FastTreeParams:
     return p
 
 
-def run_planner(case, kv_slot_map=None):
+def run_planner(case, kv_slot_map=None, backend=None):
     """Product planner on a golden case: (tree, ptrs, batch, plan, params, stdout)."""
     tree, ptrs, batch = build_tree(case["tree"])
     params = params_for(case)
     out = io.StringIO()
     with contextlib.redirect_stdout(out):
         plan = fasttree_plan(tree, ptrs, batch, case["Hkv"], case["kv_split_sizes"], case["para_threshs1"],
-                             case["para_threshs2"], params, kv_slot_map=kv_slot_map)
+                             case["para_threshs2"], params, kv_slot_map=kv_slot_map, backend=backend)
     return tree, ptrs, batch, plan, params, out.getvalue()
 
 

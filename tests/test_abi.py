@@ -74,3 +74,19 @@ def test_decode_refuses_cpu_tensors():
     with pytest.raises(AssertionError):   # mismatched q / k head dimension, as the reference asserts
         fasttree_decode(q, q[..., :16], q, q, idx, idx, idx, idx, idx, idx, idx, idx, idx, q.float(), q.float()[..., 0],
                         [0, 1], [0, 0], [16, 4], [32, 32], 0.1)
+
+
+def test_planner_header_symbols_are_exported():
+    from fasttree_hip import _plan_lib
+    text = open(os.path.join(ROOT, "include", "fasttree_plan.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(ft_plan_[a-z0-9_]+)\s*\(", text)))
+    assert names == ["ft_plan_copy", "ft_plan_create", "ft_plan_destroy", "ft_plan_size", "ft_plan_version"]
+    lib = ctypes.CDLL(_plan_lib.LIB_PATH)
+    for name in names:
+        assert hasattr(lib, name), name
+    assert set(_plan_lib.SIGNATURES) == set(names)
+    # the enum of result arrays and the Python constants agree
+    enum = re.search(r"enum \{\s*FT_PLAN_KV_ENTRIES = 0,(.*?)FT_PLAN_ARRAYS", text, flags=re.S).group(1)
+    assert len(re.findall(r"FT_PLAN_[A-Z_]+", enum)) + 1 == _plan_lib.N_ARRAYS
+    assert _plan_lib.load().ft_plan_size(None, 0) == -1

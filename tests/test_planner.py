@@ -19,12 +19,13 @@ def goldens():
     return planner_goldens()
 
 
+@pytest.mark.parametrize("backend", ["python", "native"])
 @pytest.mark.parametrize("case", PLANNER_CASES, ids=[c["name"] for c in PLANNER_CASES])
-def test_planner_matches_reference_fixture(case, goldens):
+def test_planner_matches_reference_fixture(case, backend, goldens):
     """Every list, the mutated tile sizes and the printed lines equal what the reference
-    planner produced for the same arguments."""
+    planner produced for the same arguments -- for the Python planner and for the C++ one."""
     gold = goldens[case["name"]]
-    _, _, batch, plan, params, text = run_planner(case)
+    _, _, batch, plan, params, text = run_planner(case, backend=backend)
     assert batch == gold["batch_size"]
     for name in ARRAYS:
         arr = np.asarray(getattr(plan, name), dtype=np.int32)
@@ -148,6 +149,33 @@ def test_single_child_chain_always_merges():
     p = FastTreeParams()
     p.set_q_tile_sizes([16, 4]); p.set_kv_tile_sizes([32, 32]); p.set_kv_group_num(4)
     assert _tree_heuristic(tree, p) == [0, 1, 1, 1]
+
+
+def test_native_planner_rejects_bad_trees():
+    from fasttree_hip import _plan_lib
+    tree, ptrs, batch = build_tree({"kind": "regular", "sizes": [1, 2], "lens": [8, 8]})
+    p = FastTreeParams()
+    p.set_q_tile_sizes([16, 4]); p.set_kv_tile_sizes([32, 32])
+    args = (batch, 8, [1024, 128], [132, 528], [132, 132], 0.66, 0.33, 0.1)
+    with pytest.raises(_plan_lib.FastTreePlannerError):
+        _plan_lib.plan(tree, ptrs[:-1], *args, p.TSQs, p.TSKs, 1)               # wrong prefix-sum length
+    with pytest.raises(_plan_lib.FastTreePlannerError):
+        _plan_lib.plan(tree, ptrs, *args, [0, 4], p.TSKs, 1)                    # tile size 0
+    tree[1].requests = [batch + 3]
+    with pytest.raises(_plan_lib.FastTreePlannerError):
+        _plan_lib.plan(tree, ptrs, *args, p.TSQs, p.TSKs, 1)                    # request id out of range
+
+
+@pytest.mark.parametrize("backend", ["python", "native"])
+def test_backends_agree_on_slot_maps_and_big_trees(backend):
+    case = next(c for c in PLANNER_CASES if c["name"] == "c4")
+    _, ptrs, _, plain, _, _ = run_planner(case, backend=backend)
+    perm = np.random.default_rng(5).permutation(ptrs[-1]).astype(np.int32)
+    _, _, _, mapped, _, _ = run_planner(case, kv_slot_map=perm, backend=backend)
+    assert np.array_equal(mapped.vnode_to_kv_entries[:-32], perm[plain.vnode_to_kv_entries[:-32]])
+    assert digest(np.asarray(mapped.vnode_to_kv_entries, dtype=np.int32)) == {
+        "python": digest, "native": digest}[backend](np.concatenate([perm[plain.vnode_to_kv_entries[:-32]],
+                                                                     np.full(32, -1, np.int32)]).astype(np.int32))
 
 
 def test_slot_map_is_an_indirection():
