@@ -266,6 +266,35 @@ def main():
                     "max_abs_vs_tree": float((og.float() - o.float()).abs().max())}
         del k_cache, v_cache, mo, ml
 
+    # ---- the reference's own no-sharing ablation: same kernels, same pool, a plan in which every
+    # leaf absorbs its whole path (alpha = beta = 0, gamma = 10, no KV split; run_benchmark.sh:67-81)
+    merged = None
+    if not args.no_gathered and args.workload != "c4":
+        from fasttree_hip.planner import FastTreeParams, fasttree_preparation
+        g = prob["hq"] // prob["hkv"]
+        p2 = FastTreeParams()
+        p2.set_values(0.0, 0.0, 10.0)
+        p2.set_q_tile_sizes(list(prob["q_tiles"]))
+        p2.set_kv_tile_sizes(list(prob["kv_tiles"]))
+        p2.set_kv_group_num(g)
+        aux2, assign2 = fasttree_preparation(prob["tree"], inp.KV_ptrs, prob["batch"], prob["hq"], prob["hkv"], 128,
+                                             [81920, 81920], [0, 0], [0, 0], p2, device=device,
+                                             kv_slot_map=inp.slot_map)
+        om = torch.empty_like(inp.Q)
+        ts = []
+        for i in range(13):
+            flush.zero_()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fasttree_decode(inp.Q, inp.K_pool, inp.V_pool, om, *aux2, list(p2.TSQs), list(p2.TSKs), scale)
+            e1.record()
+            e1.synchronize()
+            if i >= 3:
+                ts.append(e0.elapsed_time(e1) * 1e3)
+        merged = {"latency_us": statistics.median(ts), "merged_nodes": int(sum(assign2)),
+                  "max_abs_vs_tree": float((om.float() - o.float()).abs().max())}
+        del aux2
+
     # ---- CPU baseline: the reference's per-request gathered formulation with PyTorch ops on the host
     cpu = None
     if not args.no_cpu_baseline:
@@ -314,6 +343,7 @@ def main():
         "parity": parity,
         "gathered_hip_baseline": gathered,
         "speedup_vs_gathered": (gathered["latency_us"] / cold_med) if gathered else None,
+        "all_merged_plan_baseline": merged,
         "cpu_baseline": cpu,
         "planner_ms": prob["plan_ms"],
     }
