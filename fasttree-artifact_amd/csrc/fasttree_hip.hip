@@ -54,6 +54,12 @@ struct F16 {
     h2 v = {(_Float16)lo, (_Float16)hi};
     return __builtin_bit_cast(unsigned, v);
   }
+  // acc + lo + hi of a packed pair, in fp32
+  static __device__ __forceinline__ float add_pair(unsigned packed, float acc) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    const h2 one = {(_Float16)1.f, (_Float16)1.f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, packed), one, acc, false);
+  }
 };
 struct BF16 {
   static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
@@ -66,6 +72,11 @@ struct BF16 {
     typedef __bf16 b2 __attribute__((ext_vector_type(2)));
     b2 v = {(__bf16)lo, (__bf16)hi};
     return __builtin_bit_cast(unsigned, v);
+  }
+  static __device__ __forceinline__ float add_pair(unsigned packed, float acc) {
+    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+    const b2 one = {(__bf16)1.f, (__bf16)1.f};
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, packed), one, acc, false);
   }
 };
 
@@ -722,18 +733,19 @@ __device__ __forceinline__ void tile_step32(const WideLane& la, unsigned off, in
 
   const float neg_m = -st.m;
   float x[16];
-  float sum = 0.f;
 #pragma unroll
-  for (int j = 0; j < 16; ++j) {
-    x[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j], sc, neg_m));
-    sum += x[j];
-  }
-  st.l += sum;
+  for (int j = 0; j < 16; ++j) x[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j], sc, neg_m));
   u32x4 pf[2];
 #pragma unroll
   for (int u = 0; u < 2; ++u)
     pf[u] = u32x4{E::pack2(x[8 * u + 0], x[8 * u + 1]), E::pack2(x[8 * u + 2], x[8 * u + 3]),
                   E::pack2(x[8 * u + 4], x[8 * u + 5]), E::pack2(x[8 * u + 6], x[8 * u + 7])};
+  // the row sum is taken over the probabilities as P.V will see them (rounded to the storage
+  // type), two per instruction
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) st.l = E::add_pair(pf[u][i], st.l);
 
   FT_TIME(__builtin_amdgcn_sched_barrier(0); const unsigned long long tc2 = FT_CLOCK(); __builtin_amdgcn_sched_barrier(0);)
 #pragma unroll
