@@ -596,21 +596,26 @@ __device__ __forceinline__ void reset_state(WideState<D>& st) {
     for (int j = 0; j < 16; ++j) st.o[db][j] = 0.f;
 }
 
-// qf[ks]: row row0 + lane%32, dims 16*ks + 8*(lane/32) .. +7; zero past the vnode.
-template <int D, bool GATHERED>
-__device__ __forceinline__ void load_q_frags32(const Stage1Args& a, const VnodeView& vn, int kvh, int row0,
-                                               u32x4 (&qf)[D / 16]) {
+// Query fragments of a wave's 32 rows, loaded in two steps so that other loads can be put
+// between the two dependent ones: the address of a lane's row (needs the request id of the row,
+// one load), then the fragments.  qf[ks]: row row0 + lane%32, dims 16*ks + 8*(lane/32) .. +7;
+// zero past the vnode (src == nullptr).
+template <bool GATHERED>
+__device__ __forceinline__ const char* q_row_address32(const Stage1Args& a, const VnodeView& vn, int kvh, int row0) {
   const int lane = threadIdx.x & 63;
   const int r = row0 + (lane & 31), h = lane >> 5;
-  const bool ok = r < vn.q_len * a.g;
-  const int ri = ok ? r / a.g : 0;
-  const int rj = ok ? r - ri * a.g : 0;
-  const int64_t entry = ok ? (GATHERED ? (int64_t)(vn.q_off / a.nsplit) : (int64_t)a.q_entries[vn.q_off + ri]) : 0;
-  const char* src = a.q + 2 * (entry * a.sq0 + (int64_t)(kvh * a.g + rj) * a.sq1 + 8 * h);
+  if (r >= vn.q_len * a.g) return nullptr;
+  const int ri = r / a.g;
+  const int rj = r - ri * a.g;
+  const int64_t entry = GATHERED ? (int64_t)(vn.q_off / a.nsplit) : (int64_t)a.q_entries[vn.q_off + ri];
+  return a.q + 2 * (entry * a.sq0 + (int64_t)(kvh * a.g + rj) * a.sq1 + 8 * h);
+}
+template <int D>
+__device__ __forceinline__ void load_q_frags32(const char* src, u32x4 (&qf)[D / 16]) {
 #pragma unroll
   for (int ks = 0; ks < D / 16; ++ks) {
     u32x4 z = {0u, 0u, 0u, 0u};
-    qf[ks] = ok ? *reinterpret_cast<const u32x4*>(src + 32 * ks) : z;
+    qf[ks] = src ? *reinterpret_cast<const u32x4*>(src + 32 * ks) : z;
   }
 }
 
@@ -824,10 +829,11 @@ __device__ __forceinline__ void merge_token_groups(float* xchg, WideState<D>& st
 // (RG * TG = kWideWaves): a wave consumes the 32-token tiles t with t % TG == tg for the rows of
 // its row group, and the TG states of a row group are merged at the end.
 template <typename E, int D, bool GATHERED>
-__device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int local_vnode, int kvh, int chunk) {
+__device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int local_vnode, const VnodeView& vn,
+                                           int kvh, int chunk) {
   using W = WideGeom<D>;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  const VnodeView vn = load_vnode<GATHERED>(a, a.vnode_begin + local_vnode);
+  FT_TIME(const unsigned long long rt_entry = wall_clock64();)
   const int rows_total = vn.q_len * a.g;
   const int nsuper = (vn.kv_len + W::kTokens - 1) / W::kTokens;
 
@@ -854,8 +860,9 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
     const int my_row0 = row0 + 32 * rg;
     const bool active = rg < rgroups && my_row0 < rows_end;
 
+    // start-up chain: [request ids of the rows, slot indices] -> [Q fragments, first K/V rows]
+    const char* q_src = q_row_address32<GATHERED>(a, vn, kvh, active ? my_row0 : rows_total);
     u32x4 qf[D / 16];
-    load_q_frags32<D, GATHERED>(a, vn, kvh, active ? my_row0 : rows_total, qf);
     WideState<D> st;
     reset_state<D>(st);
     WideLane la0;
@@ -909,14 +916,15 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
       }
     };
     if (nsuper > 0) stage_indices(0);  // block uniform
+#pragma unroll
+    for (int j = 0; j < W::kAhead; ++j) issue_rows(j);
+    load_q_frags32<D>(q_src, qf);
     // nothing the compiler itself tracks (the Q fragments) may still be in flight in the loop:
     // a wait for it there would also wait for every direct load
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     // (and the compiler must see the fragments as complete, or it keeps a wait for them in the loop)
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(qf[ks]));
-#pragma unroll
-    for (int j = 0; j < W::kAhead; ++j) issue_rows(j);
     FT_TIME(unsigned long long t_start = FT_CLOCK(); unsigned long long rt_start = wall_clock64(); unsigned long long t_wait = 0, t_bar = 0, t_issue = 0, t_comp = 0; unsigned long long t_step[4] = {0, 0, 0, 0};)
     for (int super = 0; super < nsuper; ++super) {
       // publish super tile `super` to the block; the ones after it may stay in flight
@@ -945,8 +953,8 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
       FT_TIME(unsigned long long c4 = FT_CLOCK(); t_wait += c1 - c0; t_bar += c2 - c1; t_issue += c3 - c2; t_comp += c4 - c3;)
     }
     FT_TIME(if (g_timing && lane == 0) {
-      unsigned long long* out = g_timing + ((size_t)(local_vnode * a.hkv + kvh) * kWideWaves + wave) * 8;
-      out[0] = g_timing_steps ? t_step[0] : t_wait; out[1] = g_timing_steps ? t_step[1] : t_bar; out[2] = g_timing_steps ? t_step[2] : t_issue; out[3] = g_timing_steps ? t_step[3] : t_comp; out[4] = FT_CLOCK() - t_start; out[5] = nsuper;
+      unsigned long long* out = g_timing + ((size_t)blockIdx.x * kWideWaves + wave) * 8;
+      out[0] = g_timing_steps ? t_step[0] : t_wait; out[1] = g_timing_steps ? t_step[1] : t_bar; out[2] = g_timing_steps ? t_step[2] : t_issue; if (g_timing_steps != 2) out[3] = g_timing_steps ? t_step[3] : t_comp; out[4] = g_timing_steps == 2 ? rt_entry : FT_CLOCK() - t_start; out[5] = nsuper + 1000 * local_vnode + 100000 * chunk;
       out[6] = rt_start; out[7] = wall_clock64();
     })
     finish_state<D>(st);
@@ -1007,8 +1015,15 @@ __device__ __forceinline__ void narrow_attend(const Stage1Args& a, const VnodeVi
     v_addr[tb] = lds0 + N::kBytesK + vr * N::kRowBytes + 16 * ((((p & 3) >> 1) & (N::kChunks - 1)) ^ N::swz(vr)) + 8 * (p & 1);
   }
 
+  // start-up chain: [request id of the lane's row, slot indices] -> [Q fragments, first K/V rows].
+  // Fragment ks of a lane: row row0 + p, dims 32*ks + 8*c .. +7; zero past the vnode.
+  const char* q_src = nullptr;
+  if (row0 + p < vn.q_len * a.g) {
+    const int r = row0 + p, ri = r / a.g, rj = r - ri * a.g;
+    const int64_t entry = GATHERED ? (int64_t)(vn.q_off / a.nsplit) : (int64_t)a.q_entries[vn.q_off + ri];
+    q_src = a.q + 2 * (entry * a.sq0 + (int64_t)(kvh * a.g + rj) * a.sq1 + 8 * c);
+  }
   u32x4 qf[1][KS];
-  load_q_frags<D, 1, GATHERED>(a, vn, kvh, row0, qf);
   reset_state<D, 1>(st);
   if (tile0 < ntiles) {
     // slot indices of tokens [idx_base, idx_base + kIdxCap) of the run
@@ -1049,14 +1064,19 @@ __device__ __forceinline__ void narrow_attend(const Stage1Args& a, const VnodeVi
       }
     };
     stage_indices(tile0 * kTileTokens);
+    issue(tile0, false);
+    issue(tile0, true);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      u32x4 z = {0u, 0u, 0u, 0u};
+      qf[0][ks] = q_src ? *reinterpret_cast<const u32x4*>(q_src + 64 * ks) : z;
+    }
     // nothing the compiler itself tracks may still be in flight below: a wait for it would
     // also wait for every direct load
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     // (and the compiler must see the fragments as complete, or it keeps a wait for them in the loop)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[0][ks]));
-    issue(tile0, false);
-    issue(tile0, true);
     for (int tile = tile0; tile < ntiles; tile += tstride) {
       const int next = tile + tstride;
       const bool more = next < ntiles;
@@ -1221,29 +1241,40 @@ __global__ void __launch_bounds__(kWideBlock) stage1_narrow_kernel(Stage1Args a)
 // itself (they are few) and takes the one whose rank is `target`.  Block uniform.
 constexpr int kMaxRanked = kWideBlock;
 template <bool GATHERED>
-__device__ __forceinline__ int wide_vnode_of_rank(const Stage1Args& a, char* smem, int target) {
+__device__ __forceinline__ int wide_vnode_of_rank(const Stage1Args& a, char* smem, int target, VnodeView& view) {
   const int n = a.vnode_count;
-  if (n < 2 || n > kMaxRanked) return target;
+  if (n < 2 || n > kMaxRanked) {
+    view = load_vnode<GATHERED>(a, a.vnode_begin + target);
+    return target;
+  }
   unsigned long long* cost = reinterpret_cast<unsigned long long*>(smem);
-  int* found = reinterpret_cast<int*>(cost + kMaxRanked);
+  VnodeView* views = reinterpret_cast<VnodeView*>(cost + kMaxRanked);
+  int* found = reinterpret_cast<int*>(views + kMaxRanked);
   const int tid = threadIdx.x;
   unsigned long long mine = 0;
   if (tid < n) {
     const VnodeView vn = load_vnode<GATHERED>(a, a.vnode_begin + tid);
     mine = (unsigned long long)(unsigned)(vn.q_len * a.g) * (unsigned)vn.kv_len;
     cost[tid] = mine;
+    views[tid] = vn;  // the block's own vnode is among them: no second trip to memory for it
   }
   __syncthreads();
   if (tid < n) {
     int rank = 0;
-    for (int j = 0; j < n; ++j) {
-      const unsigned long long c = cost[j];
-      rank += (c > mine || (c == mine && j < tid)) ? 1 : 0;
+    // (costs in batches of eight, so that the reads of a batch are in flight together)
+    for (int j0 = 0; j0 < n; j0 += 8) {
+      unsigned long long c[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) c[i] = cost[min(j0 + i, n - 1)];
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        rank += (j0 + i < n && (c[i] > mine || (c[i] == mine && j0 + i < tid))) ? 1 : 0;
     }
     if (rank == target) *found = tid;
   }
   __syncthreads();
   const int v = *found;
+  view = views[v];
   __syncthreads();  // the ranking area is reused as the staging ring
   return v;
 }
@@ -1254,6 +1285,7 @@ __device__ __forceinline__ int wide_vnode_of_rank(const Stage1Args& a, char* sme
 template <typename E, int D, bool GATHERED>
 __global__ void __launch_bounds__(kWideBlock, 512 / kWideBlock) stage1_fused_kernel(Stage1Args a) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
+  FT_TIME(if (g_timing && g_timing_steps == 2 && (threadIdx.x & 63) == 0) g_timing[((size_t)blockIdx.x * kWideWaves + (threadIdx.x >> 6)) * 8 + 3] = wall_clock64();)
   const int wide_blocks = a.vnode_count * a.wide_chunks * a.hkv;
   const int wide_index = blockIdx.x, narrow_index = (int)blockIdx.x - wide_blocks;
   const bool is_wide = (int)blockIdx.x < wide_blocks;
@@ -1261,9 +1293,15 @@ __global__ void __launch_bounds__(kWideBlock, 512 / kWideBlock) stage1_fused_ker
     const int per_rank = a.wide_chunks * a.hkv;
     const int rank = wide_index / per_rank;
     const int rest = wide_index - rank * per_rank;
-    const int chunk = rest / a.hkv;
-    const int local_vnode = wide_vnode_of_rank<GATHERED>(a, smem, rank);
-    wide_block<E, D, GATHERED>(a, smem, local_vnode, rest - chunk * a.hkv, chunk);
+    // Launch slot `rest / hkv` of a rank serves chunk (slot + rank / 2) % chunks.  Consecutive
+    // blocks of one kv head go round robin to the four shader engines of an XCD, strictly in
+    // order (a block waits for its engine even when others have room); without the rotation an
+    // engine would only ever get first chunks, which run longer than last ones.
+    const int slot = rest / a.hkv;
+    const int chunk = (slot + (rank >> 1)) % a.wide_chunks;
+    VnodeView vn;
+    const int local_vnode = wide_vnode_of_rank<GATHERED>(a, smem, rank, vn);
+    wide_block<E, D, GATHERED>(a, smem, local_vnode, vn, rest - slot * a.hkv, chunk);
   } else {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int share = a.narrow_share;
