@@ -1367,34 +1367,36 @@ __global__ void __launch_bounds__(kBlock) stage2_kernel(Stage2Args a) {
   for (int base = 0; base < n; base += LPH) {
     const int cnt = min(LPH, n - base);
     int my_row = -1;
+    if (gl < cnt) my_row = a.nsplit > 0 ? off + base + gl : a.req_entries[off + base + gl];
+    // Rows in batches of kBatch, all loads of a batch issued before the first is used (the rows
+    // are in bounds whatever their weight; a zero weight discards the row's contents).  The
+    // first batch is requested together with the log-sum-exp values, not after them: both
+    // depend on the row indices only.
+    constexpr int kBatch = 8;
+    f32x4 part[kBatch];
+    auto request = [&](int i0) {
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) {
+        const int ri = __shfl(my_row, min(i0 + j, cnt - 1), LPH);
+        part[j] = *reinterpret_cast<const f32x4*>(a.mid_o + (int64_t)ri * a.so0 + (int64_t)head * a.so1 + 4 * gl);
+      }
+    };
     float my_lse = -INFINITY;
-    if (gl < cnt) {
-      my_row = a.nsplit > 0 ? off + base + gl : a.req_entries[off + base + gl];
-      my_lse = a.mid_lse[(int64_t)my_row * a.sl0 + head];
-    }
+    if (gl < cnt) my_lse = a.mid_lse[(int64_t)my_row * a.sl0 + head];
+    request(0);
     const float m_new = fmaxf(m_run, group_max<LPH>(my_lse));
     const float w = (my_lse == -INFINITY) ? 0.f : __expf(my_lse - m_new);
     const float keep = (m_run == -INFINITY) ? 0.f : __expf(m_run - m_new);
     l_run = l_run * keep + group_sum<LPH>(w);
     acc *= keep;
     m_run = m_new;
-    // rows in batches of kBatch: all loads of a batch are issued before the first is used (the
-    // rows are in bounds whatever their weight; a zero weight discards the row's contents)
-    constexpr int kBatch = 8;
     for (int i0 = 0; i0 < cnt; i0 += kBatch) {
-      f32x4 part[kBatch];
-      float wi[kBatch];
+      if (i0 > 0) request(i0);
 #pragma unroll
       for (int j = 0; j < kBatch; ++j) {
-        const int i = min(i0 + j, cnt - 1);
-        wi[j] = (i0 + j < cnt) ? __shfl(w, i, LPH) : 0.f;
-        const int ri = __shfl(my_row, i, LPH);
-        part[j] = *reinterpret_cast<const f32x4*>(a.mid_o + (int64_t)ri * a.so0 + (int64_t)head * a.so1 + 4 * gl);
-      }
+        const float wi = (i0 + j < cnt) ? __shfl(w, min(i0 + j, cnt - 1), LPH) : 0.f;
 #pragma unroll
-      for (int j = 0; j < kBatch; ++j) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc[e] += (wi[j] != 0.f) ? part[j][e] * wi[j] : 0.f;
+        for (int e = 0; e < 4; ++e) acc[e] += (wi != 0.f) ? part[j][e] * wi : 0.f;
       }
     }
   }
