@@ -336,3 +336,69 @@ def test_runs_on_a_side_stream_and_unsupported_inputs_raise(device):
     bad = torch.zeros(batch, 8, 48, dtype=torch.float16, device=device)
     with pytest.raises(AssertionError):
         fasttree_decode(bad, bad, bad, bad, *aux, [16, 4], [32, 32], 0.1)
+
+
+def _plan_and_check(device, sizes, lens, hq, hkv, d, q_tiles, splits, what, dtype=torch.float16, seed=11, sample=None,
+                    thr=((1, 1), (1, 1))):
+    tree, ptrs, batch = build_tree({"kind": "regular", "sizes": sizes, "lens": lens})
+    inp = make_decode_inputs(tree, hq, hkv, d, device=device, dtype=dtype, seed=seed, shuffle_slots=True)
+    params = FastTreeParams()
+    params.set_values(0.66, 0.33, 0.1); params.set_q_tile_sizes(list(q_tiles)); params.set_kv_tile_sizes([32, 32])
+    params.set_kv_group_num(hq // hkv)
+    aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, hq, hkv, d, list(splits), list(thr[0]), list(thr[1]), params,
+                                  device=device, kv_slot_map=inp.slot_map)
+    o = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, list(params.TSQs), [32, 32], 1.0 / math.sqrt(d))
+    _dense_check(tree, inp, o, what, sample, dtype=dtype)
+    return aux
+
+
+@pytest.mark.gpu
+def test_wide_vnodes_in_row_chunks_and_uneven_tails(device):
+    """Wide vnodes of 3 x 128 + 52 query rows (four blocks per vnode and kv head, the last one
+    with a token split), runs that are no multiple of a tile, and a staged index window that is
+    refilled (runs longer than 2048 tokens)."""
+    _announce("row chunks")
+    aux = _plan_and_check(device, [1, 3, 327], [2500, 77, 5], 16, 4, 128, [109, 4], [4096, 4096], "row chunks",
+                          sample=list(range(0, 327, 5)))
+    assert aux[11][0] >= 3  # the wide phase exists
+    _plan_and_check(device, [1, 109], [2077, 31], 8, 8, 64, [109, 16], [4096, 64], "row chunks mha d64",
+                    sample=list(range(0, 109, 3)))
+
+
+@pytest.mark.gpu
+def test_more_wide_vnodes_than_the_ranking_holds(device):
+    """More than 256 wide vnodes: blocks take them in plan order instead of ranking them."""
+    _announce("many wide vnodes")
+    aux = _plan_and_check(device, [1, 300, 1800], [40, 70, 9], 32, 8, 128, [16, 4], [1024, 128], "many wide vnodes",
+                          sample=list(range(0, 1800, 37)))
+    assert aux[11][0] > 256
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("batch", [1, 5, 40, 150])
+def test_few_long_narrow_vnodes_are_shared_between_waves(batch, device):
+    """Few requests with long private runs: 8, 4 or 2 waves share a narrow vnode (all-narrow
+    launch and, with a wide root, the fused launch), incl. runs longer than the 256-token index
+    window and a last tile of one token."""
+    _announce("shared narrow vnodes", batch)
+    _plan_and_check(device, [1, batch], [64, 1441], 16, 1, 128, [16, 1], [4096, 4096], f"shared narrow {batch} g16",
+                    dtype=torch.bfloat16)
+    _plan_and_check(device, [1, batch], [700, 545], 32, 8, 128, [64, 4], [4096, 4096], f"shared narrow {batch} fused")
+
+
+@pytest.mark.gpu
+def test_narrow_vnode_wider_than_its_tile_argument_with_shared_waves(device):
+    """Tile arguments that call a 40-row vnode narrow (q tile 4 x g 4): several 16-row passes
+    per vnode while waves share it."""
+    _announce("narrow passes")
+    tree, ptrs, batch = build_tree({"kind": "regular", "sizes": [1, 10], "lens": [333, 50]})
+    inp = make_decode_inputs(tree, 32, 8, 128, device=device, dtype=torch.float16, seed=4, shuffle_slots=True)
+    params = FastTreeParams()
+    params.set_q_tile_sizes([16, 4]); params.set_kv_tile_sizes([32, 32]); params.set_kv_group_num(4)
+    aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, 32, 8, 128, [4096, 4096], [1, 1], [1, 1], params,
+                                  device=device, kv_slot_map=inp.slot_map)
+    # everything as one narrow range of 4-request tiles: the 10-request root vnode has 40 rows
+    aux = list(aux)
+    aux[11], aux[12] = [0, sum(aux[11])], [0, 0]
+    o = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, [4, 4], [32, 32], 1.0 / math.sqrt(128))
+    _dense_check(tree, inp, o, "narrow passes")
