@@ -1239,6 +1239,12 @@ __global__ void __launch_bounds__(kWideBlock) stage1_narrow_kernel(Stage1Args a)
 // vnodes in order of decreasing work (query rows x tokens) is longest-job-first list scheduling:
 // the machine does not end on a late start of a long block.  Every block ranks the wide vnodes
 // itself (they are few) and takes the one whose rank is `target`.  Block uniform.
+//
+// On the way, neighbours in the vnode list that attend the same KV run with adjoining scratch
+// rows -- the query tiles the planner cut one node into -- are joined into one work item of at
+// most `cap` query rows (what the blocks of one vnode serve in a single pass): a tile of 16
+// requests x 4 heads fills only half of a block's rows, and two such tiles would stage the same
+// run twice.  The first vnode of a group carries the group; the others become empty items.
 constexpr int kMaxRanked = kWideBlock;
 template <bool GATHERED>
 __device__ __forceinline__ int wide_vnode_of_rank(const Stage1Args& a, char* smem, int target, VnodeView& view) {
@@ -1247,34 +1253,84 @@ __device__ __forceinline__ int wide_vnode_of_rank(const Stage1Args& a, char* sme
     view = load_vnode<GATHERED>(a, a.vnode_begin + target);
     return target;
   }
-  unsigned long long* cost = reinterpret_cast<unsigned long long*>(smem);
-  VnodeView* views = reinterpret_cast<VnodeView*>(cost + kMaxRanked);
-  int* found = reinterpret_cast<int*>(views + kMaxRanked);
+  // keys[u]: work of vnode u in 24 bits (a float's exponent and leading mantissa bits), then
+  // 255 - u: larger key = earlier, no two equal; 0 for a vnode that is not the head of a group
+  unsigned* keys = reinterpret_cast<unsigned*>(smem);
+  VnodeView* views = reinterpret_cast<VnodeView*>(keys + kMaxRanked);
+  int* group_q_len = reinterpret_cast<int*>(views + kMaxRanked);
+  unsigned long long* joined = reinterpret_cast<unsigned long long*>(group_q_len + kMaxRanked);  // one bit per vnode
+  int* found = reinterpret_cast<int*>(joined + kMaxRanked / 64);
   const int tid = threadIdx.x;
-  unsigned long long mine = 0;
-  if (tid < n) {
-    const VnodeView vn = load_vnode<GATHERED>(a, a.vnode_begin + tid);
-    mine = (unsigned long long)(unsigned)(vn.q_len * a.g) * (unsigned)vn.kv_len;
-    cost[tid] = mine;
-    views[tid] = vn;  // the block's own vnode is among them: no second trip to memory for it
-  }
+  if (tid < n) views[tid] = load_vnode<GATHERED>(a, a.vnode_begin + tid);  // the block's own vnode is among them
+  if (tid == 0) *found = -1;
   __syncthreads();
+  // bit u: vnode u continues vnode u - 1 (same run, adjoining scratch rows)
+  bool joins = false;
+  if (tid > 0 && tid < n) {
+    const VnodeView& p = views[tid - 1];
+    const VnodeView& c = views[tid];
+    joins = p.kv_base == c.kv_base && p.kv_len == c.kv_len && p.q_off + p.q_len == c.q_off;
+  }
+  const unsigned long long wave_bits = __ballot(joins);
+  if ((tid & 63) == 0) joined[tid >> 6] = wave_bits;
+  __syncthreads();
+  unsigned mine = 0;
   if (tid < n) {
+    // first and last vnode of the chain of joined vnodes that holds this one
+    int first = tid;
+    for (int w = tid >> 6, hi = tid & 63; w >= 0; --w, hi = 63) {
+      const unsigned long long stops = ~joined[w] & (hi == 63 ? ~0ull : ((2ull << hi) - 1));
+      if (stops) {
+        first = 64 * w + 63 - __builtin_clzll(stops);
+        break;
+      }
+    }
+    int last = n - 1;
+    for (int u = tid + 1, w = u >> 6; w < (n + 63) / 64; ++w, u = 64 * w) {
+      const unsigned long long stops = ~joined[w] & (~0ull << (u & 63));
+      if (stops) {
+        last = min(n, 64 * w + __builtin_ctzll(stops)) - 1;
+        break;
+      }
+    }
+    // groups of m vnodes from the start of the chain; the chain's first vnode is a full query tile
+    const long long cap = (long long)kWideRows * a.wide_chunks;
+    const long long tile_rows = max(1LL, (long long)views[first].q_len * a.g);
+    const int m = (int)max(1LL, cap / tile_rows);
+    const int head = first + (tid - first) / m * m;
+    int q_len = 0;
+    if (head == tid) {
+      const VnodeView& tail = views[min(last, head + m - 1)];
+      q_len = tail.q_off + tail.q_len - views[tid].q_off;
+      const float work = (float)q_len * (float)a.g * (float)views[tid].kv_len;
+      mine = ((__builtin_bit_cast(unsigned, work) >> 7) << 8) | (unsigned)(255 - tid);
+    }
+    group_q_len[tid] = q_len;
+  }
+  keys[tid] = mine;  // all kMaxRanked entries: the vector reads below run over the padding
+  __syncthreads();
+  if (mine != 0) {
     int rank = 0;
-    // (costs in batches of eight, so that the reads of a batch are in flight together)
-    for (int j0 = 0; j0 < n; j0 += 8) {
-      unsigned long long c[8];
+    for (int j0 = 0; j0 < n; j0 += 16) {  // (keys past n are 0 and count for nothing)
+      u32x4 k[4];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) c[i] = cost[min(j0 + i, n - 1)];
+      for (int i = 0; i < 4; ++i) k[i] = *reinterpret_cast<const u32x4*>(keys + j0 + 4 * i);
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
-        rank += (j0 + i < n && (c[i] > mine || (c[i] == mine && j0 + i < tid))) ? 1 : 0;
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) rank += k[i][e] > mine ? 1 : 0;
     }
     if (rank == target) *found = tid;
   }
   __syncthreads();
   const int v = *found;
+  if (v < 0) {  // more ranks than groups: an empty item
+    view = VnodeView{0, 0, 0, 0};
+    __syncthreads();
+    return 0;
+  }
   view = views[v];
+  view.q_len = group_q_len[v];
   __syncthreads();  // the ranking area is reused as the staging ring
   return v;
 }
