@@ -324,11 +324,9 @@ __device__ __forceinline__ void tile_step(const char* ldsK, const char* ldsV, in
 }
 
 // One wave attends NQB*16 query rows to tokens [tile0*32, ...) in steps of tile_step_n tiles,
-// staging each tile in its own LDS area.  Rows travel global -> registers -> LDS.  With DEEP,
-// the rows of the next two tiles and the slot indices of the two after those are in flight while
-// a tile is consumed, so a short run (the common leaf vnode) has all of its loads issued at
-// once instead of paying one memory round trip per tile; without it, one tile is in flight.
-template <typename E, int D, int NQB, bool GATHERED, bool DEEP = false>
+// staging each tile in its own LDS area.  Rows travel global -> registers -> LDS; the next tile
+// is in flight while a tile is consumed.  (Used for head_dim 256 only.)
+template <typename E, int D, int NQB, bool GATHERED>
 __device__ __forceinline__ void wave_attend(const Stage1Args& a, const VnodeView& vn, int kvh, int row0,
                                             int tile0, int tile_step_n, char* lds, WaveState<D, NQB>& st) {
   using G = TileGeom<D>;
@@ -378,44 +376,18 @@ __device__ __forceinline__ void wave_attend(const Stage1Args& a, const VnodeView
     wave_lds_fence();
   };
 
-  if constexpr (!DEEP) {
-    int slot[G::kLoads];
-    u32x4 kreg[G::kLoads], vreg[G::kLoads];
-    load_slots(tile0, slot);
-    load_rows(slot, kreg, vreg);
-    for (int tile = tile0; tile < ntiles; tile += tile_step_n) {
-      stage(kreg, vreg);
-      if (tile + tile_step_n < ntiles) {
-        load_slots(tile + tile_step_n, slot);
-        load_rows(slot, kreg, vreg);
-      }
-      tile_step<E, D, NQB>(ldsK, ldsV, vn.kv_len - tile * kTileTokens, a.scale_log2, qf, st);
-      wave_lds_fence();
+  int slot[G::kLoads];
+  u32x4 kreg[G::kLoads], vreg[G::kLoads];
+  load_slots(tile0, slot);
+  load_rows(slot, kreg, vreg);
+  for (int tile = tile0; tile < ntiles; tile += tile_step_n) {
+    stage(kreg, vreg);
+    if (tile + tile_step_n < ntiles) {
+      load_slots(tile + tile_step_n, slot);
+      load_rows(slot, kreg, vreg);
     }
-  } else {
-    // even tiles use set 0, odd tiles set 1 (tile numbering relative to tile0, step tile_step_n)
-    int slot0[G::kLoads], slot1[G::kLoads];
-    u32x4 k0[G::kLoads], v0[G::kLoads], k1[G::kLoads], v1[G::kLoads];
-    const int dt = tile_step_n;
-    load_slots(tile0, slot0);
-    load_slots(tile0 + dt, slot1);
-    load_rows(slot0, k0, v0);
-    load_rows(slot1, k1, v1);
-    load_slots(tile0 + 2 * dt, slot0);
-    load_slots(tile0 + 3 * dt, slot1);
-    for (int tile = tile0; tile < ntiles; tile += 2 * dt) {
-      stage(k0, v0);
-      load_rows(slot0, k0, v0);                 // tile + 2*dt
-      load_slots(tile + 4 * dt, slot0);
-      tile_step<E, D, NQB>(ldsK, ldsV, vn.kv_len - tile * kTileTokens, a.scale_log2, qf, st);
-      wave_lds_fence();
-      if (tile + dt >= ntiles) break;
-      stage(k1, v1);
-      load_rows(slot1, k1, v1);                 // tile + 3*dt
-      load_slots(tile + 5 * dt, slot1);
-      tile_step<E, D, NQB>(ldsK, ldsV, vn.kv_len - (tile + dt) * kTileTokens, a.scale_log2, qf, st);
-      wave_lds_fence();
-    }
+    tile_step<E, D, NQB>(ldsK, ldsV, vn.kv_len - tile * kTileTokens, a.scale_log2, qf, st);
+    wave_lds_fence();
   }
   finish_state<D, NQB>(st);
 }
@@ -1465,13 +1437,20 @@ __global__ void __launch_bounds__(kBlock) stage2_kernel(Stage2Args a) {
 // ---------------------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------------------
+constexpr int kMaxDevices = 64;
+inline int current_device() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) (void)hipGetLastError();
+  return dev >= 0 && dev < kMaxDevices ? dev : 0;
+}
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 template <typename E, int D, int NQB, bool SPLIT, bool GATHERED>
 int launch_stage1_inst(const Stage1Args& a, int hkv, hipStream_t stream) {
   const size_t lds = (size_t)kWavesPerBlock * TileGeom<D>::kBytes;
   auto kern = stage1_kernel<E, D, NQB, SPLIT, GATHERED>;
-  static bool configured = false;  // raising the dynamic LDS limit is idempotent
+  static bool configured_on[kMaxDevices] = {};  // raising the dynamic LDS limit is idempotent
+  bool& configured = configured_on[current_device()];
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
       (void)hipGetLastError();
@@ -1509,7 +1488,8 @@ int launch_stage1_fused(const Stage1Args& a0, hipStream_t stream) {
   constexpr size_t kNarrowLds = (size_t)kWideWaves * NarrowGeom<D>::kLds;
   constexpr size_t lds = kWideLds > kNarrowLds ? kWideLds : kNarrowLds;
   auto kern = stage1_fused_kernel<E, D, GATHERED>;
-  static bool configured = false;  // raising the dynamic LDS limit is idempotent
+  static bool configured_on[kMaxDevices] = {};  // raising the dynamic LDS limit is idempotent
+  bool& configured = configured_on[current_device()];
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
       (void)hipGetLastError();
@@ -1539,7 +1519,8 @@ int launch_stage1_narrow(const Stage1Args& a0, hipStream_t stream) {
   a.narrow_share = narrow_share_for(blocks);
   auto kern = stage1_narrow_kernel<E, D, GATHERED>;
   const size_t lds = (size_t)a.narrow_share * NarrowGeom<D>::kLds;
-  static bool configured = false;  // raising the dynamic LDS limit is idempotent
+  static bool configured_on[kMaxDevices] = {};  // raising the dynamic LDS limit is idempotent
+  bool& configured = configured_on[current_device()];
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             kWideWaves * NarrowGeom<D>::kLds) != hipSuccess) {
