@@ -44,6 +44,8 @@ WORKLOADS = {
     "c2": ([1, 64], [4096, 256], 32, 8, "fp16"),
     "c3": ([1, 10, 400], [4000, 400, 40], 32, 8, "fp16"),
     "c4": ([1, 2048], [512, 1024], 32, 8, "bf16"),
+    # seeded irregular tree (5 levels, fan-out U[1,8], lengths log-uniform [16,2048], <= 1024 leaves); sizes = seed
+    "c5": (0, None, 64, 8, "fp16"),
 }
 
 # Planner arguments.  "reference" = the values the reference bench passes
@@ -74,7 +76,8 @@ def build_problem(name, preset, device, seed=0):
 
     sizes, lens, hq, hkv, dt = WORKLOADS[name]
     dtype = {"fp16": torch.float16, "bf16": torch.bfloat16}[dt]
-    tree, ptrs, batch = build_tree({"kind": "regular", "sizes": sizes, "lens": lens})
+    spec = {"kind": "irregular", "seed": sizes} if lens is None else {"kind": "regular", "sizes": sizes, "lens": lens}
+    tree, ptrs, batch = build_tree(spec)
     big = ptrs[-1] * hkv * 128 > (1 << 28)
     inp = make_decode_inputs(tree, hq, hkv, 128, device=device, dtype=dtype, seed=seed, shuffle_slots=True,
                              host_rng=not big)
@@ -330,7 +333,8 @@ def main():
         "dtype": "f16" if prob["dtype"] == "fp16" else "bf16",
         "data": "synthetic",
         "config": {"workload": {"c1": "2-level tree 1x1024 + 16x128", "c2": "2-level tree 1x4096 + 64x256", "c3": "3-level tree N=[1,10,400] C=[4000,400,40]",
-                                "c4": "2-level tree 1x512 + 2048x1024"}[args.workload]
+                                "c4": "2-level tree 1x512 + 2048x1024",
+                                "c5": "irregular 5-level tree, seed 0"}[args.workload]
                    + f", {prob['hq']}q/{prob['hkv']}kv heads, head_dim 128, {prob['dtype']}, paged pool (page 1, shuffled), "
                    + f"{prob['batch']} requests", "planner_preset": args.preset,
                    "q_tiles": prob["q_tiles"], "vnodes": [int(x) for x in nums], "scratch_rows": int(rows)},
