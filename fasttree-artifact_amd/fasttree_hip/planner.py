@@ -421,6 +421,28 @@ def fasttree_plan(
     )
 
 
+def narrow_vnodes_longest_first(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, phase_node_offsets, group):
+    """The four per-vnode lists with the vnodes of the second phase in order of decreasing work.
+
+    A vnode is the tuple (kv_offs[v], kv_lens[v], q_offs[v], q_lens[v]); nothing else refers to
+    a vnode by its position (the per-request lists of kernel_bench/fasttree.py:233-244 name
+    scratch rows, not vnodes), so any order within a phase computes the same result.  The
+    decode kernel hands the narrow vnodes to the machine in list order, each to one wave that
+    walks the run tile by tile: a long run that starts last is what the launch then waits for.
+    Work is counted as KV tokens times passes of 16 query rows; equal work keeps the planner's
+    order.  The first phase is left alone (the kernel ranks its vnodes itself).
+    """
+    lists = [np.array(x, dtype=np.int32, copy=True) for x in (kv_offs, kv_lens, q_offs, q_lens)]
+    begin, count = int(phase_node_offsets[1]), int(phase_node_nums[1])
+    if count > 1:
+        part = slice(begin, begin + count)
+        passes = (lists[3][part].astype(np.int64) * int(group) + 15) // 16
+        order = np.argsort(-(lists[1][part].astype(np.int64) * passes), kind="stable")
+        for x in lists:
+            x[part] = x[part][order]
+    return tuple(lists)
+
+
 def fasttree_preparation(
     tree_info,
     KV_ptrs,
@@ -435,6 +457,7 @@ def fasttree_preparation(
     *,
     device="cuda",
     kv_slot_map=None,
+    launch_order=True,
 ):
     """Drop-in for kernel_bench/fasttree.py:99-296: plan on the host, then place the nine
     int32 index arrays and the two fp32 partial-result buffers on ``device``.
@@ -444,7 +467,9 @@ def fasttree_preparation(
     req_to_vnode_offs, req_to_vnode_lens, mid_o, mid_lse, phase_node_nums,
     phase_node_offsets), node_assignments)``.  The keyword-only arguments do not exist
     in the reference: ``device`` defaults to the reference's hard-wired "cuda";
-    ``kv_slot_map`` is described in :func:`fasttree_plan`.
+    ``kv_slot_map`` is described in :func:`fasttree_plan`; ``launch_order`` lists the narrow
+    vnodes longest first (:func:`narrow_vnodes_longest_first`) instead of in the reference's
+    tree order.
     """
     import torch
 
@@ -458,15 +483,19 @@ def fasttree_preparation(
         return host.to(device)
 
     rows = plan.num_rows
+    vnodes = (plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens)
+    if launch_order:
+        vnodes = narrow_vnodes_longest_first(*vnodes, plan.phase_node_nums, plan.phase_node_offsets,
+                                             max(1, num_qo_heads // num_kv_heads))
     mid_o = torch.empty((rows, num_qo_heads, head_dim), dtype=torch.float32, device=device)
     mid_lse = torch.empty((rows, num_qo_heads), dtype=torch.float32, device=device)
     aux = (
         put(plan.vnode_to_kv_entries),
-        put(plan.vnode_to_kv_offs),
-        put(plan.vnode_to_kv_lens),
+        put(vnodes[0]),
+        put(vnodes[1]),
         put(plan.vnode_to_q_entries),
-        put(plan.vnode_to_q_offs),
-        put(plan.vnode_to_q_lens),
+        put(vnodes[2]),
+        put(vnodes[3]),
         put(plan.req_to_vnode_entries),
         put(plan.req_to_vnode_offs),
         put(plan.req_to_vnode_lens),

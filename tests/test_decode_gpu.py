@@ -120,6 +120,27 @@ def test_baseline_configs_against_dense_oracle(name, preset, device):
     assert_parity(o, ref.reshape(batch, hq, 128), f"{name}/{preset} vs torch fp32")
 
 
+def test_vnode_order_within_a_phase_does_not_change_the_result(device):
+    """Narrow vnodes longest first (the default of fasttree_preparation) against the planner's
+    own order: a vnode is computed the same way wherever it stands in its phase."""
+    _announce("vnode order")
+    tree, ptrs, batch = build_tree({"kind": "irregular", "seed": 3})
+    inp = make_decode_inputs(tree, 32, 8, 128, device=device, dtype=torch.float16, seed=11, shuffle_slots=True)
+    outs = []
+    for launch_order in (False, True):
+        params = FastTreeParams()
+        params.set_values(0.66, 0.33, 0.1); params.set_q_tile_sizes([16, 4]); params.set_kv_tile_sizes([32, 32])
+        params.set_kv_group_num(4)
+        aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, 32, 8, 128, [1024, 128], [132, 528], [132, 132], params,
+                                      device=device, kv_slot_map=inp.slot_map, launch_order=launch_order)
+        wide = aux[11][0]
+        lens = aux[2].cpu().numpy()[wide:].astype(np.int64) * ((aux[5].cpu().numpy()[wide:].astype(np.int64) * 4 + 15) // 16)
+        assert launch_order == bool((np.diff(lens) <= 0).all()), "the irregular tree's own order is not sorted"
+        outs.append(_decode(inp.Q, inp.K_pool, inp.V_pool, aux, [16, 4], [32, 32], 1.0 / math.sqrt(128)))
+    assert torch.equal(outs[0], outs[1])
+    print(_dense_check(tree, inp, outs[1], "vnode order", list(range(0, batch, 5))), flush=True)
+
+
 @pytest.mark.parametrize("seed", [0, 1, 2])
 def test_deep_irregular_tree(seed, device):
     """C5: 5 levels, fan-out U[1,8], lengths log-uniform [16,2048], <= 1024 leaves, GQA 8."""

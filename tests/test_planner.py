@@ -130,6 +130,25 @@ def test_plan_invariants(name):
         assert rows == sorted(rows) and all(plan.vnode_to_q_entries[x] == r for x in rows)
 
 
+@pytest.mark.parametrize("name", ["kat1", "c3", "c5_seed0", "rand17"])
+def test_longest_first_order_is_a_permutation_within_the_narrow_phase(name):
+    """The launch order keeps the vnode tuples, moves none across the phase boundary, and puts
+    the narrow vnodes in order of decreasing tokens x passes with ties in planner order."""
+    from fasttree_hip.planner import narrow_vnodes_longest_first
+    case = next(c for c in PLANNER_CASES if c["name"] == name)
+    tree, ptrs, batch, plan, params, _ = run_planner(case)
+    group = case["Hq"] // case["Hkv"]
+    before = list(zip(plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens))
+    after = list(zip(*(x.tolist() for x in narrow_vnodes_longest_first(
+        plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens,
+        plan.phase_node_nums, plan.phase_node_offsets, group))))
+    wide = plan.phase_node_nums[0]
+    assert after[:wide] == before[:wide]
+    work = lambda v: v[1] * ((v[3] * group + 15) // 16)
+    assert after[wide:] == sorted(before[wide:], key=lambda v: -work(v))  # (sorted() is stable)
+    assert list(plan.vnode_to_kv_lens) == [v[1] for v in before], "the plan itself is not touched"
+
+
 def test_ablation_extremes():
     """gamma = +10 with alpha = beta = 0 merges every node into its leaf path (one vnode per
     request over its whole path); gamma = -10 never merges."""
