@@ -59,7 +59,8 @@ MEASURED_TRAFFIC = {("c3", "mi355x", "stage1"): 148.8e6, ("c4", "mi355x", "stage
 
 PRESETS = {
     "reference": dict(q_tiles=None, kv_tiles=(32, 32), kv_splits=(1024, 128), thr1=(132, 528), thr2=(132, 132)),
-    "mi355x": dict(q_tiles="wide", kv_tiles=(32, 32), kv_splits=(1024, 128), thr1=(256, 1024), thr2=(256, 256)),
+    "mi355x": dict(q_tiles=None, kv_tiles=(32, 32), kv_splits=(1024, 128), thr1=(256, 1024), thr2=(256, 256)),
+    "wide": dict(q_tiles="wide", kv_tiles=(32, 32), kv_splits=(1024, 128), thr1=(256, 1024), thr2=(256, 256)),
 }
 
 

@@ -132,6 +132,7 @@ struct Stage1Args {
   int narrow_share;                // waves that share one narrow vnode: 1, 2, 4 or 8
   int wide_rows;                   // query rows the planner's tile gives a wide vnode (host hint for wide_chunks)
   int wide_chunks;                 // blocks per (wide vnode, kv head); block c serves row pieces c, c + wide_chunks, ..
+  int block_slots;                 // blocks of the fused kernel the device runs at a time
   int g;
   int hkv;
   float scale_log2;  // sm_scale * log2(e)
@@ -1236,9 +1237,11 @@ __device__ __forceinline__ int wide_vnode_of_rank(const Stage1Args& a, char* sme
   if (tid < n) views[tid] = load_vnode<GATHERED>(a, a.vnode_begin + tid);  // the block's own vnode is among them
   if (tid == 0) *found = -1;
   __syncthreads();
-  // bit u: vnode u continues vnode u - 1 (same run, adjoining scratch rows)
+  // bit u: vnode u continues vnode u - 1 (same run, adjoining scratch rows).  Nothing is joined
+  // while there are no more blocks than compute units: two half-filled blocks side by side
+  // finish sooner than one full block.
   bool joins = false;
-  if (tid > 0 && tid < n) {
+  if (tid > 0 && tid < n && 2LL * n * a.hkv * a.wide_chunks > a.block_slots) {
     const VnodeView& p = views[tid - 1];
     const VnodeView& c = views[tid];
     joins = p.kv_base == c.kv_base && p.kv_len == c.kv_len && p.q_off + p.q_len == c.q_off;
@@ -1467,7 +1470,7 @@ int launch_stage1_inst(const Stage1Args& a, int hkv, hipStream_t stream) {
 // three quarters of the wave slots (8 per compute unit).  With far fewer vnodes than slots the
 // waves would each walk a long run alone, one memory round trip per tile; with the slots nearly
 // full the runs are limited by memory bandwidth already and sharing only adds barriers.
-inline int narrow_share_for(int64_t items) {
+inline int wave_slots() {
   static int slots = 0;
   if (slots == 0) {
     int dev = 0, cus = 0;
@@ -1477,6 +1480,10 @@ inline int narrow_share_for(int64_t items) {
     }
     slots = cus * kWaveSlotsPerCu;
   }
+  return slots;
+}
+inline int narrow_share_for(int64_t items) {
+  const int slots = wave_slots();
   int share = 1;
   while (share < kWideWaves && 4 * items * (2 * share) <= 3 * (int64_t)slots) share *= 2;
   return share;
@@ -1503,6 +1510,7 @@ int launch_stage1_fused(const Stage1Args& a0, hipStream_t stream) {
   const int per_block = kWideWaves / a.narrow_share;
   const int64_t narrow_blocks = (narrow_items + per_block - 1) / per_block;
   a.wide_chunks = std::max(1, std::min(8, (a.wide_rows + kWideRows - 1) / kWideRows));
+  a.block_slots = wave_slots() / kWideWaves;
   const int64_t blocks = (int64_t)a.vnode_count * a.wide_chunks * a.hkv + narrow_blocks;
   if (blocks == 0) return FT_OK;
   if (blocks > INT32_MAX) return FT_ERR_ARGUMENT;

@@ -421,26 +421,60 @@ def fasttree_plan(
     )
 
 
-def narrow_vnodes_longest_first(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, phase_node_offsets, group):
-    """The four per-vnode lists with the vnodes of the second phase in order of decreasing work.
+#: A first-phase vnode of at most LIGHT_VNODE_ROWS query rows and LIGHT_VNODE_WORK query rows x
+#: KV tokens is launched with the second phase when the first phase alone has more blocks than
+#: WIDE_BLOCK_SLOTS, the number an MI355X runs at a time (256 compute units x 2); see
+#: :func:`vnodes_in_launch_order`.
+LIGHT_VNODE_WORK = int(os.environ.get("FASTTREE_LIGHT_VNODE_WORK", "4096"))
+LIGHT_VNODE_ROWS = 64
+WIDE_BLOCK_SLOTS = 512
+
+
+def vnodes_in_launch_order(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, phase_node_offsets, group,
+                           num_kv_heads=None, light_work=None):
+    """The four per-vnode lists and the two phase lists, rearranged for the decode kernels.
 
     A vnode is the tuple (kv_offs[v], kv_lens[v], q_offs[v], q_lens[v]); nothing else refers to
     a vnode by its position (the per-request lists of kernel_bench/fasttree.py:233-244 name
-    scratch rows, not vnodes), so any order within a phase computes the same result.  The
-    decode kernel hands the narrow vnodes to the machine in list order, each to one wave that
-    walks the run tile by tile: a long run that starts last is what the launch then waits for.
-    Work is counted as KV tokens times passes of 16 query rows; equal work keeps the planner's
-    order.  The first phase is left alone (the kernel ranks its vnodes itself).
+    scratch rows, not vnodes), and the kernels compute a vnode of any number of query rows in
+    either phase, so the order within a phase and the phase a vnode is launched with change the
+    schedule, not the result.  Two changes against the reference's order (fasttree.py:246-259):
+
+    * light first-phase vnodes -- at most :data:`LIGHT_VNODE_ROWS` query rows and query rows x
+      KV tokens at most ``light_work`` (default :data:`LIGHT_VNODE_WORK`) -- move to the second
+      phase, provided the first phase has more blocks (vnodes x ``num_kv_heads``) than the
+      machine runs at a time (:data:`WIDE_BLOCK_SLOTS`; always, when ``num_kv_heads`` is None).
+      A first-phase vnode gets a block of four waves with a staging ring for long runs, two
+      blocks per compute unit; a second-phase vnode gets one wave that serves 16 rows per
+      pass, eight or more per compute unit.  Short runs under a few dozen rows are bound by
+      memory latency, not by arithmetic: when there are more of them than block slots, they
+      finish sooner with more of them in flight; when there are fewer, a block's four waves
+      finish one sooner than a single wave's passes do.
+    * the second phase is listed in order of decreasing work (KV tokens x passes of 16 rows;
+      equal work keeps the order).  The kernel hands these vnodes to the machine in list order,
+      each to one wave that walks its run tile by tile: a long run that starts last is what the
+      launch then waits for.
+
+    The order within the first phase is left alone (the kernel ranks those vnodes itself).
+    Returns ``(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, phase_node_offsets)``.
     """
+    light_work = LIGHT_VNODE_WORK if light_work is None else light_work
     lists = [np.array(x, dtype=np.int32, copy=True) for x in (kv_offs, kv_lens, q_offs, q_lens)]
-    begin, count = int(phase_node_offsets[1]), int(phase_node_nums[1])
-    if count > 1:
-        part = slice(begin, begin + count)
-        passes = (lists[3][part].astype(np.int64) * int(group) + 15) // 16
-        order = np.argsort(-(lists[1][part].astype(np.int64) * passes), kind="stable")
-        for x in lists:
-            x[part] = x[part][order]
-    return tuple(lists)
+    first, count0, count1 = int(phase_node_offsets[0]), int(phase_node_nums[0]), int(phase_node_nums[1])
+    if first != 0 or int(phase_node_offsets[1]) != count0:
+        raise ValueError("the phases must be adjoining ranges starting at vnode 0")
+    rows = lists[3].astype(np.int64) * int(group)
+    tokens = lists[1].astype(np.int64)
+    index = np.arange(count0 + count1)
+    light = (index < count0) & (rows * tokens <= light_work) & (rows <= LIGHT_VNODE_ROWS)
+    if num_kv_heads is not None and count0 * int(num_kv_heads) <= WIDE_BLOCK_SLOTS:
+        light[:] = False
+    wide = index[(index < count0) & ~light]
+    narrow = np.concatenate([index[light], index[count0:]])
+    work = tokens[narrow] * ((rows[narrow] + 15) // 16)
+    narrow = narrow[np.argsort(-work, kind="stable")]
+    order = np.concatenate([wide, narrow])
+    return (*(x[order] for x in lists), [len(wide), len(narrow)], [0, len(wide)])
 
 
 def fasttree_preparation(
@@ -467,9 +501,9 @@ def fasttree_preparation(
     req_to_vnode_offs, req_to_vnode_lens, mid_o, mid_lse, phase_node_nums,
     phase_node_offsets), node_assignments)``.  The keyword-only arguments do not exist
     in the reference: ``device`` defaults to the reference's hard-wired "cuda";
-    ``kv_slot_map`` is described in :func:`fasttree_plan`; ``launch_order`` lists the narrow
-    vnodes longest first (:func:`narrow_vnodes_longest_first`) instead of in the reference's
-    tree order.
+    ``kv_slot_map`` is described in :func:`fasttree_plan`; ``launch_order`` arranges the vnodes
+    for the kernels (:func:`vnodes_in_launch_order`) instead of leaving them in the reference's
+    order.
     """
     import torch
 
@@ -483,10 +517,10 @@ def fasttree_preparation(
         return host.to(device)
 
     rows = plan.num_rows
-    vnodes = (plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens)
+    vnodes = (plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens,
+              plan.phase_node_nums, plan.phase_node_offsets)
     if launch_order:
-        vnodes = narrow_vnodes_longest_first(*vnodes, plan.phase_node_nums, plan.phase_node_offsets,
-                                             max(1, num_qo_heads // num_kv_heads))
+        vnodes = vnodes_in_launch_order(*vnodes, max(1, num_qo_heads // num_kv_heads), num_kv_heads)
     mid_o = torch.empty((rows, num_qo_heads, head_dim), dtype=torch.float32, device=device)
     mid_lse = torch.empty((rows, num_qo_heads), dtype=torch.float32, device=device)
     aux = (
@@ -501,7 +535,7 @@ def fasttree_preparation(
         put(plan.req_to_vnode_lens),
         mid_o,
         mid_lse,
-        plan.phase_node_nums,
-        plan.phase_node_offsets,
+        list(vnodes[4]),
+        list(vnodes[5]),
     )
     return aux, plan.node_assignments

@@ -1,0 +1,178 @@
+"""Kernel micro-benchmark with the command line of kernel_bench/benchmark.py:241-275.
+
+    python benchmark.py --load_file_path trees/c3.txt --num_qo_heads 32 --num_kv_heads 8 \\
+        --q_tile_size_per_phase 16,4 --choice all
+
+Engines (``--choice``): ``fasttree`` is the tree decode (planner + the two HIP stages);
+``flash_attn`` is the decode without prefix sharing over the per-request gathered cache
+``[B, max_seqlen, Hkv, D]`` (the layout of kernel_bench/flash_attn_wrap.py:36-70), here a HIP
+kernel of this library, and it is the result the tree decode is checked against with the
+reference's criterion ``allclose(rtol=1e-2, atol=1e-2)`` (kernel_bench/benchmark.py:216-220).
+The reference's other engines (SGLang Triton, FlashInfer, DeFT) are Triton / CUDA libraries and
+have no counterpart here.
+
+Timing follows the method of ``triton.testing.do_bench`` as the reference calls it
+(kernel_bench/benchmark.py:35,59): per-call device events, a 256 MB buffer cleared before every
+call, a repetition count sized for about 100 ms, the median reported in milliseconds.
+``--mi355x`` replaces the H100 defaults of the query tiles (64,16, right for 32/32 heads only) and
+of the parallelism thresholds with the ones for MI355X: tiles of 64 // g and 16 // g requests, as
+the reference's sweep picks them per GQA ratio (kernel_bench/run_benchmark.sh:46-53), and
+thresholds for 256 compute units instead of 132; explicit options win over it.
+"""
+import argparse
+import os
+import sys
+
+import torch
+
+sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), ".."))
+
+from fasttree_hip import planner as _planner  # noqa: E402
+from fasttree_hip.decode import fasttree_decode, gathered_decode  # noqa: E402
+from fasttree_hip.inputs import qkv_preparation  # noqa: E402
+from fasttree_hip.kv_tree import retrive_from_file  # noqa: E402
+from fasttree_hip.planner import FastTreeParams, fasttree_preparation  # noqa: E402
+
+QUANTILES = [0.5, 0.2, 0.8]
+
+
+def do_bench(fn, quantiles=QUANTILES, warmup=25, rep=100):
+    """Milliseconds per call at the given quantiles; cold L2 (a 256 MB buffer is cleared before
+    every call), one event pair per call."""
+    fn()
+    torch.cuda.synchronize()
+    cache = torch.empty(256 << 20, dtype=torch.int8, device="cuda")
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(5):
+        cache.zero_()
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    estimate = start.elapsed_time(end) / 5
+    n_warmup = max(1, int(warmup / estimate))
+    n_repeat = max(1, int(rep / estimate))
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(n_repeat)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(n_repeat)]
+    for _ in range(n_warmup):
+        fn()
+    for i in range(n_repeat):
+        cache.zero_()
+        starts[i].record()
+        fn()
+        ends[i].record()
+    torch.cuda.synchronize()
+    times = torch.tensor([s.elapsed_time(e) for s, e in zip(starts, ends)], dtype=torch.float64)
+    return torch.quantile(times, torch.tensor(quantiles, dtype=torch.float64)).tolist()
+
+
+def main(args):
+    num_qo_heads, num_kv_heads, head_dim = args.num_qo_heads, args.num_kv_heads, args.head_dim
+    group = num_qo_heads // num_kv_heads
+    dtype = torch.float16
+    defaults = dict(q_tile_size_per_phase="64,16", para_threshs1="132,528", para_threshs2="132,132")
+    if args.mi355x:
+        defaults = dict(q_tile_size_per_phase=f"{max(1, 64 // group)},{max(1, 16 // group)}",
+                        para_threshs1="256,1024", para_threshs2="256,256")
+    ints = lambda text: list(map(int, text.split(",")))
+    Q_TILE_SIZE_PER_PHASE = ints(args.q_tile_size_per_phase or defaults["q_tile_size_per_phase"])
+    KV_TILE_SIZE_PER_PHASE = ints(args.kv_tile_size_per_phase)
+    KV_SPLIT_SIZES = ints(args.kv_split_sizes)
+    para_threshs1 = ints(args.para_threshs1 or defaults["para_threshs1"])
+    para_threshs2 = ints(args.para_threshs2 or defaults["para_threshs2"])
+
+    params = FastTreeParams()
+    params.set_values(args.alpha, args.beta, args.gamma)
+    params.set_q_tile_sizes(Q_TILE_SIZE_PER_PHASE)
+    params.set_kv_tile_sizes(KV_TILE_SIZE_PER_PHASE)
+    params.set_kv_group_num(group)
+
+    tree_info = retrive_from_file(args.load_file_path)
+    Q, K_cache, V_cache, cache_seqlens, K_tree_tensor, V_tree_tensor, KV_ptrs = qkv_preparation(
+        tree_info, num_qo_heads, num_kv_heads, head_dim, "cuda", dtype)
+    batch_size = Q.shape[0]
+    sm_scale = 1.0 / (head_dim ** 0.5)
+    results = {}
+
+    def run_and_bench(func, name):
+        if args.signature:
+            name = args.signature
+        out = func()
+        ms, _, _ = do_bench(func, quantiles=QUANTILES)
+        print(f"{name} time:", ms, flush=True)
+        results[name] = ms
+        return out
+
+    out_flash_attn = None
+    out_tree_attn = None
+
+    if args.choice in ["flash_attn", "all"]:
+        out_gathered = torch.empty(batch_size, num_qo_heads, head_dim, device="cuda", dtype=dtype)
+        kv_split = 512
+        nsplit = (K_cache.shape[1] + kv_split - 1) // kv_split
+        mid_o = torch.empty((batch_size * nsplit, num_qo_heads, head_dim), dtype=torch.float32, device="cuda")
+        mid_lse = torch.empty((batch_size * nsplit, num_qo_heads), dtype=torch.float32, device="cuda")
+
+        def call_gathered():
+            gathered_decode(Q, K_cache, V_cache, cache_seqlens, out_gathered, sm_scale, kv_split, mid_o, mid_lse)
+            return out_gathered
+
+        out_flash_attn = run_and_bench(call_gathered, "flash attn").cpu()
+
+    if args.choice in ["fasttree", "all"]:
+        _planner.VERBOSE = not args.quiet
+        fasttree_aux, node_assignment = fasttree_preparation(
+            tree_info, KV_ptrs, batch_size, num_qo_heads, num_kv_heads, head_dim,
+            KV_SPLIT_SIZES, para_threshs1, para_threshs2, params)
+        if args.fasttree_heuristic_path:
+            with open(args.fasttree_heuristic_path, "w") as file:
+                for i in range(len(tree_info)):
+                    file.write(f"Node {i}: parent {tree_info[i].parent}, assignment {node_assignment[i]}\n")
+        out_tree = torch.empty(batch_size, num_qo_heads, head_dim, device="cuda", dtype=dtype)
+        # (the tiles the planner ended with; they differ from the command line's only when its
+        # second pass collapsed the phases, kernel_bench/fasttree.py:181-186)
+        q_tiles, kv_tiles = list(params.TSQs), list(params.TSKs)
+
+        def call_tree_attn():
+            fasttree_decode(Q, K_tree_tensor, V_tree_tensor, out_tree, *fasttree_aux, q_tiles, kv_tiles, sm_scale)
+            return out_tree
+
+        out_tree_attn = run_and_bench(call_tree_attn, "fasttree attn").cpu()
+
+    if out_flash_attn is not None and out_tree_attn is not None:
+        ok = torch.allclose(out_flash_attn, out_tree_attn, rtol=1e-2, atol=1e-2)
+        print("fasttree attn Check passed!" if ok else "fasttree attn Check failed!", flush=True)
+        err = (out_flash_attn.float() - out_tree_attn.float()).abs()
+        results["max_abs"] = err.max().item()
+        results["worst_request_mean_abs"] = err.mean(dim=(1, 2)).max().item()
+        results["check"] = bool(ok)
+        print(f"max abs difference: {results['max_abs']:.3e}, worst request mean abs: "
+              f"{results['worst_request_mean_abs']:.3e}", flush=True)
+    return results
+
+
+def build_parser():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--load_file_path", type=str, required=True)
+    parser.add_argument("--alpha", type=float, default=0.66)
+    parser.add_argument("--beta", type=float, default=0.33)
+    parser.add_argument("--gamma", type=float, default=0.1)
+    parser.add_argument("--q_tile_size_per_phase", type=str, default=None, help="default 64,16")
+    parser.add_argument("--kv_tile_size_per_phase", type=str, default="32,32")
+    parser.add_argument("--kv_split_sizes", type=str, default="1024,128")
+    parser.add_argument("--para_threshs1", type=str, default=None, help="default 132,528")
+    parser.add_argument("--para_threshs2", type=str, default=None, help="default 132,132")
+    parser.add_argument("--fasttree_heuristic_path", type=str, default=None)
+    parser.add_argument("--num_qo_heads", type=int, default=32)
+    parser.add_argument("--num_kv_heads", type=int, default=32)
+    parser.add_argument("--head_dim", type=int, default=128)
+    parser.add_argument("--signature", type=str, default=None)
+    parser.add_argument("--choice", type=str, choices=["flash_attn", "fasttree", "all"], default="all")
+    parser.add_argument("--mi355x", action="store_true", default=False,
+                        help="query tiles and parallelism thresholds for MI355X instead of the H100 defaults")
+    parser.add_argument("--quiet", action="store_true", default=False, help="do not print the planner's lines")
+    return parser
+
+
+if __name__ == "__main__":
+    main(build_parser().parse_args())

@@ -130,23 +130,38 @@ def test_plan_invariants(name):
         assert rows == sorted(rows) and all(plan.vnode_to_q_entries[x] == r for x in rows)
 
 
-@pytest.mark.parametrize("name", ["kat1", "c3", "c5_seed0", "rand17"])
-def test_longest_first_order_is_a_permutation_within_the_narrow_phase(name):
-    """The launch order keeps the vnode tuples, moves none across the phase boundary, and puts
-    the narrow vnodes in order of decreasing tokens x passes with ties in planner order."""
-    from fasttree_hip.planner import narrow_vnodes_longest_first
+@pytest.mark.parametrize("light_work", [0, 4096, 1 << 40])
+@pytest.mark.parametrize("name", ["kat1", "c3", "c5_seed0", "rand17", "shape07_h32_8"])
+def test_launch_order_is_a_permutation_of_the_vnodes(name, light_work):
+    """The launch order keeps the vnode tuples; first-phase vnodes of at most light_work rows x
+    tokens join the second phase, which is listed by decreasing tokens x passes with ties in the
+    previous order; the other first-phase vnodes keep their order."""
+    from fasttree_hip.planner import vnodes_in_launch_order
     case = next(c for c in PLANNER_CASES if c["name"] == name)
     tree, ptrs, batch, plan, params, _ = run_planner(case)
     group = case["Hq"] // case["Hkv"]
     before = list(zip(plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens))
-    after = list(zip(*(x.tolist() for x in narrow_vnodes_longest_first(
+    *lists, nums, offs = vnodes_in_launch_order(
         plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens,
-        plan.phase_node_nums, plan.phase_node_offsets, group))))
+        plan.phase_node_nums, plan.phase_node_offsets, group, light_work=light_work)
+    after = list(zip(*(x.tolist() for x in lists)))
     wide = plan.phase_node_nums[0]
-    assert after[:wide] == before[:wide]
+    light = lambda v: v[1] * v[3] * group <= light_work and v[3] * group <= 64
     work = lambda v: v[1] * ((v[3] * group + 15) // 16)
-    assert after[wide:] == sorted(before[wide:], key=lambda v: -work(v))  # (sorted() is stable)
+    stay = [v for v in before[:wide] if not light(v)]
+    move = [v for v in before[:wide] if light(v)]
+    assert nums == [len(stay), len(before) - len(stay)] and offs == [0, len(stay)]
+    assert after[:nums[0]] == stay
+    assert after[nums[0]:] == sorted(move + before[wide:], key=lambda v: -work(v))  # (sorted() is stable)
+    assert sorted(after) == sorted(before)
     assert list(plan.vnode_to_kv_lens) == [v[1] for v in before], "the plan itself is not touched"
+    if light_work == 0:
+        assert nums == list(plan.phase_node_nums)
+    # with the number of kv heads given, nothing moves unless the first phase oversubscribes the machine
+    *_, nums_few, _ = vnodes_in_launch_order(
+        plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens,
+        plan.phase_node_nums, plan.phase_node_offsets, group, 1, light_work=light_work)
+    assert nums_few == (nums if wide > 512 else list(plan.phase_node_nums))
 
 
 def test_ablation_extremes():
