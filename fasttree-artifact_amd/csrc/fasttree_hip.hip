@@ -1438,6 +1438,40 @@ __global__ void __launch_bounds__(kBlock) stage2_kernel(Stage2Args a) {
 }
 
 // ---------------------------------------------------------------------------------------
+// The step's new K and V rows into the pools (one launch for both)
+// ---------------------------------------------------------------------------------------
+struct StoreArgs {
+  const char* k_new;
+  const char* v_new;
+  int64_t kn0, kn1, vn0, vn1;  // element strides of the new rows [tokens, Hkv, D]
+  const void* loc;             // pool slot per token, int32 or int64
+  int loc_is_int64;
+  char* k_pool;
+  char* v_pool;
+  int64_t sk0, sk1, sv0, sv1;
+  int64_t num_slots;
+  int tokens, hkv, chunks;     // chunks = 16-byte pieces per (token, head) row
+};
+
+// One thread moves 16 bytes of a K row and the same 16 bytes of the V row.  A token whose slot
+// lies outside the pool is skipped.
+__global__ void __launch_bounds__(256) store_kv_kernel(StoreArgs a) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int per_token = a.hkv * a.chunks;
+  const int64_t token = i / per_token;
+  if (token >= a.tokens) return;
+  const int rest = (int)(i - token * per_token);
+  const int head = rest / a.chunks, chunk = rest - head * a.chunks;
+  const int64_t slot = a.loc_is_int64 ? static_cast<const int64_t*>(a.loc)[token]
+                                      : (int64_t) static_cast<const int32_t*>(a.loc)[token];
+  if (slot < 0 || slot >= a.num_slots) return;
+  const u32x4 kx = *reinterpret_cast<const u32x4*>(a.k_new + 2 * (token * a.kn0 + head * a.kn1) + 16 * chunk);
+  const u32x4 vx = *reinterpret_cast<const u32x4*>(a.v_new + 2 * (token * a.vn0 + head * a.vn1) + 16 * chunk);
+  *reinterpret_cast<u32x4*>(a.k_pool + 2 * (slot * a.sk0 + head * a.sk1) + 16 * chunk) = kx;
+  *reinterpret_cast<u32x4*>(a.v_pool + 2 * (slot * a.sv0 + head * a.sv1) + 16 * chunk) = vx;
+}
+
+// ---------------------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------------------
 constexpr int kMaxDevices = 64;
@@ -1835,6 +1869,33 @@ int ft_gathered_decode(const void* q, const void* k_cache, const void* v_cache,
   b.o = static_cast<char*>(o); b.oo0 = oo0; b.oo1 = oo1;
   b.batch = batch_size; b.hq = num_qo_heads; b.nsplit = nsplit;
   return launch_stage2(b, head_dim, dtype, stream);
+}
+
+int ft_store_kv(const void* k_new, const void* v_new, int64_t kn0, int64_t kn1, int64_t vn0, int64_t vn1,
+                const void* out_cache_loc, int loc_is_int64, int num_tokens,
+                void* k_pool, void* v_pool, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+                int64_t num_slots, int num_kv_heads, int head_dim, int dtype, ft_stream_t stream) {
+  if (dtype != FT_DTYPE_F16 && dtype != FT_DTYPE_BF16) return FT_ERR_DTYPE;
+  if (head_dim < 8 || head_dim % 8 != 0 || head_dim > 1024) return FT_ERR_HEAD_DIM;
+  if (num_tokens == 0) return FT_OK;
+  if (!k_new || !v_new || !out_cache_loc || !k_pool || !v_pool) return FT_ERR_NULL_POINTER;
+  if (num_tokens < 0 || num_kv_heads < 1 || num_kv_heads > 65535 || num_slots < 0) return FT_ERR_ARGUMENT;
+  if (!aligned16(k_new) || !aligned16(v_new) || !aligned16(k_pool) || !aligned16(v_pool) ||
+      (kn0 | kn1 | vn0 | vn1 | sk0 | sk1 | sv0 | sv1) % 8 != 0)
+    return FT_ERR_ALIGNMENT;
+  if (kn0 < 0 || kn1 < 0 || vn0 < 0 || vn1 < 0 || sk0 < 0 || sk1 < 0 || sv0 < 0 || sv1 < 0) return FT_ERR_ARGUMENT;
+  StoreArgs a{};
+  a.k_new = static_cast<const char*>(k_new); a.v_new = static_cast<const char*>(v_new);
+  a.kn0 = kn0; a.kn1 = kn1; a.vn0 = vn0; a.vn1 = vn1;
+  a.loc = out_cache_loc; a.loc_is_int64 = loc_is_int64 ? 1 : 0;
+  a.k_pool = static_cast<char*>(k_pool); a.v_pool = static_cast<char*>(v_pool);
+  a.sk0 = sk0; a.sk1 = sk1; a.sv0 = sv0; a.sv1 = sv1;
+  a.num_slots = num_slots; a.tokens = num_tokens; a.hkv = num_kv_heads; a.chunks = head_dim / 8;
+  const int64_t threads = (int64_t)num_tokens * num_kv_heads * a.chunks;
+  const int64_t blocks = (threads + 255) / 256;
+  if (blocks > INT32_MAX) return FT_ERR_ARGUMENT;
+  hipLaunchKernelGGL(store_kv_kernel, dim3((unsigned)blocks, 1, 1), dim3(256, 1, 1), 0, stream, a);
+  return hipGetLastError() == hipSuccess ? FT_OK : FT_ERR_LAUNCH;
 }
 
 }  // extern "C"

@@ -34,6 +34,8 @@ SIGNATURES = {
                   + [_P, c_int64, c_int64, _P, c_int64] + [_P] * 4 + [c_int] * 4 + [c_float, c_int, _P]),
     "ft_gathered_decode": (c_int, [_P, _P, _P, _P, _P] + [c_int64] * 4 + [c_int] * 6 + [c_float]
                            + [_P, _P, c_int, _P]),
+    "ft_store_kv": (c_int, [_P, _P] + [c_int64] * 4 + [_P, c_int, c_int, _P, _P] + [c_int64] * 5
+                    + [c_int, c_int, c_int, _P]),
 }
 
 _lib = None

@@ -158,3 +158,39 @@ def gathered_decode(q, k_cache, v_cache, cache_seqlens, o, sm_scale, kv_split=51
     )
     _lib.check(rc, "ft_gathered_decode")
     return mid_o, mid_lse
+
+
+def store_kv_cache(cache_k, cache_v, out_cache_loc, k_buffer, v_buffer):
+    """``k_buffer[out_cache_loc] = cache_k; v_buffer[out_cache_loc] = cache_v`` in one launch on
+    the current stream: the two indexed assignments of SGLang v0.2.13's
+    ``RadixAttention.store_kv_cache``, the step that precedes the decode in the hook
+    (fasttree_sglang_plugin_v0_2_13/plugin.py:26).
+
+    ``cache_k`` / ``cache_v`` are ``[tokens, Hkv, D]`` (or ``[tokens, Hkv * D]``), ``out_cache_loc``
+    int32 or int64 pool slots.  A slot outside the pool is skipped, not wrapped.
+    """
+    import torch
+
+    _need_gpu(cache_k, cache_v, out_cache_loc, k_buffer, v_buffer)
+    hkv, d = k_buffer.shape[1], k_buffer.shape[2]
+    if v_buffer.shape[1:] != k_buffer.shape[1:] or v_buffer.dtype != k_buffer.dtype:
+        raise _lib.FastTreeLibraryError("k_buffer and v_buffer must have the same heads, head size and dtype")
+    cache_k = cache_k.view(-1, hkv, d)
+    cache_v = cache_v.view(-1, hkv, d)
+    if cache_k.dtype != k_buffer.dtype or cache_v.dtype != k_buffer.dtype:
+        raise _lib.FastTreeLibraryError("the new rows must have the pools' dtype")
+    _need_inner_contiguous(cache_k, cache_v, k_buffer, v_buffer)
+    n = cache_k.shape[0]
+    if cache_v.shape[0] != n or out_cache_loc.numel() != n:
+        raise _lib.FastTreeLibraryError("cache_k, cache_v and out_cache_loc must name the same number of tokens")
+    if out_cache_loc.dtype not in (torch.int32, torch.int64) or not out_cache_loc.is_contiguous():
+        raise _lib.FastTreeLibraryError("out_cache_loc must be a contiguous int32 or int64 tensor")
+    lib = _lib.load()
+    rc = lib.ft_store_kv(
+        cache_k.data_ptr(), cache_v.data_ptr(), cache_k.stride(0), cache_k.stride(1), cache_v.stride(0), cache_v.stride(1),
+        out_cache_loc.data_ptr(), int(out_cache_loc.dtype == torch.int64), n,
+        k_buffer.data_ptr(), v_buffer.data_ptr(), k_buffer.stride(0), k_buffer.stride(1),
+        v_buffer.stride(0), v_buffer.stride(1), min(k_buffer.shape[0], v_buffer.shape[0]), hkv, d,
+        _dtype_code(k_buffer), _stream_handle(k_buffer),
+    )
+    _lib.check(rc, "ft_store_kv")

@@ -29,8 +29,8 @@ class FastTreeMetadata:
     """Planner hyper-parameters plus the device buffers one decode step reads (metadata.py:5-66).
 
     Buffers are allocated once at their maxima; a plan fills prefixes of them.  The defaults are
-    the reference's, including ``para_threshs1=(132, 132)`` / ``para_threshs2=(132, 528)``.
-    On MI355X pass ``TSQs=(256 // g, 16 // g)`` and thresholds scaled to 256 compute units.
+    the reference's, including ``para_threshs1=(132, 132)`` / ``para_threshs2=(132, 528)``
+    (132 = compute units of an H100; an MI355X has 256).
     """
 
     def __init__(
@@ -50,6 +50,7 @@ class FastTreeMetadata:
         max_vnodes: int = 16384,
         max_vnode_to_q_entries: int = 81920,
         max_batch_size: int = 8192,
+        fused_store: bool = False,
     ):
         self.num_qo_heads = num_qo_heads
         self.num_kv_heads = num_kv_heads
@@ -62,6 +63,9 @@ class FastTreeMetadata:
         self.kv_split_sizes = kv_split_sizes
         self.para_threshs1 = para_threshs1
         self.para_threshs2 = para_threshs2
+        #: not in the reference: the hook writes the step's K/V rows with this library's single
+        #: launch instead of calling the layer's ``store_kv_cache``
+        self.fused_store = fused_store
 
         def ints(n):
             return torch.empty(n, dtype=torch.int32, device=device)
@@ -92,20 +96,26 @@ class FastTreeMetadata:
 def decode_forward_fasttree(self, q, k, v, input_metadata):
     """``RadixAttention.decode_forward`` replacement (plugin.py:15-51).
 
-    Stores the step's K/V rows through the layer's own ``store_kv_cache``, then runs the tree
-    decode with the pool buffers, ``req_to_token`` as the flat KV-index array and the metadata
-    bound to ``input_metadata.fasttree``.  The output shape for ``qk_head_dim != v_head_dim``
+    Stores the step's K/V rows through the layer's own ``store_kv_cache`` (or, with
+    ``FastTreeMetadata(fused_store=True)``, with one launch of this library for both pools), then
+    runs the tree decode with the pool buffers, ``req_to_token`` as the flat KV-index array and
+    the metadata bound to ``input_metadata.fasttree``.  The output shape for ``qk_head_dim != v_head_dim``
     follows the reference literally (plugin.py:22-23).
     """
-    from .decode import fasttree_decode
+    from .decode import fasttree_decode, store_kv_cache
 
     if self.qk_head_dim != self.v_head_dim:
         o = q.new_empty((q.shape[-1], self.tp_q_head_num * self.v_head_dim))
     else:
         o = torch.empty_like(q)
-    self.store_kv_cache(k, v, input_metadata)
-
     meta = input_metadata.fasttree
+    if getattr(meta, "fused_store", False):
+        store_kv_cache(k, v, input_metadata.out_cache_loc,
+                       input_metadata.token_to_kv_pool.get_key_buffer(self.layer_id),
+                       input_metadata.token_to_kv_pool.get_value_buffer(self.layer_id))
+    else:
+        self.store_kv_cache(k, v, input_metadata)
+
     fasttree_decode(
         q.view(-1, self.tp_q_head_num, self.qk_head_dim),
         input_metadata.token_to_kv_pool.get_key_buffer(self.layer_id),

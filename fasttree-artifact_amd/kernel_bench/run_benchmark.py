@@ -14,6 +14,7 @@ decode, and performance normalised to the best engine of the row
 import argparse
 import contextlib
 import io
+import math
 import os
 import sys
 
@@ -100,6 +101,14 @@ def write_table(rows, path):
             fh.write(f"| {r['tree']} | {r['heads']} | {r['preset']} | {r['flash_attn']:.4f} | {r['naive']:.4f} | {r['no_greedy']:.4f} | "
                      f"{r['fasttree']:.4f} | {r['flash_attn'] / r['fasttree']:.2f} | {norm} | {'passed' if r['check'] else 'FAILED'} | "
                      f"{r['max_abs']:.1e} | {r['mean_abs']:.1e} |\n")
+        fh.write("\n")
+        for preset in sorted({r["preset"] for r in rows}):
+            part = [r for r in rows if r["preset"] == preset]
+            geo = math.exp(sum(math.log(r["flash_attn"] / r["fasttree"]) for r in part) / len(part))
+            best = sum(1 for r in part if r["fasttree"] <= 1.05 * min(r[e] for e in engines))
+            fh.write(f"Preset `{preset}`: {len(part)} cases, geometric-mean speed-up of the tree decode over the gathered "
+                     f"decode {geo:.2f}x; the tree decode is the fastest engine (within 5 %) in {best} of them; "
+                     f"{sum(1 for r in part if not r['check'])} failed the allclose check.\n\n")
 
 
 def main(argv=None):

@@ -131,6 +131,19 @@ int ft_gathered_decode(const void* q, const void* k_cache, const void* v_cache,
                        int head_dim, int kv_split, float sm_scale,
                        float* mid_o, float* mid_lse, int dtype, ft_stream_t stream);
 
+/*
+ * The decode step's new K and V rows [num_tokens, Hkv, D] written to the pools at the slots
+ * out_cache_loc[t] (int32, or int64 when loc_is_int64), both tensors in one launch on `stream`:
+ * the two indexed assignments of SGLang v0.2.13's RadixAttention.store_kv_cache, which the hook
+ * runs immediately before the decode (sglang_v0.2.13_bench/fasttree_sglang_plugin_v0_2_13/
+ * plugin.py:26).  A token whose slot is outside [0, num_slots) is skipped.  Strides in elements,
+ * multiples of 8; D a multiple of 8.  Work enqueued later on the same stream sees the rows.
+ */
+int ft_store_kv(const void* k_new, const void* v_new, int64_t kn0, int64_t kn1, int64_t vn0, int64_t vn1,
+                const void* out_cache_loc, int loc_is_int64, int num_tokens,
+                void* k_pool, void* v_pool, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+                int64_t num_slots, int num_kv_heads, int head_dim, int dtype, ft_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -22,7 +22,7 @@ def declared_symbols():
 def test_header_symbols_are_exported():
     names = declared_symbols()
     assert names == ["ft_decode", "ft_error_string", "ft_gathered_decode", "ft_stage1", "ft_stage1_phases", "ft_stage2",
-                     "ft_version"]
+                     "ft_store_kv", "ft_version"]
     lib = ctypes.CDLL(_lib.LIB_PATH)
     for name in names:
         assert hasattr(lib, name), name
@@ -60,6 +60,18 @@ def test_argument_checks_return_codes_without_touching_a_device():
         _lib.check(-3, "x")
     with pytest.raises(_lib.FastTreeLibraryError):
         _lib.check(-5, "x")
+
+    def store(ptr=0x1000, tokens=3, head_dim=128, dtype=0, stride=1024, heads=8):
+        return lib.ft_store_kv(ptr, ptr, stride, 128, stride, 128, ptr, 0, tokens, ptr, ptr, stride, 128, stride, 128,
+                               100, heads, head_dim, dtype, None)
+
+    assert store(tokens=0) == 0
+    assert store(ptr=null) == -1
+    assert store(dtype=3) == -2
+    assert store(head_dim=12) == -3
+    assert store(ptr=0x1008) == -5
+    assert store(stride=1028) == -5
+    assert store(tokens=-1) == -6 and store(heads=0) == -6 and store(stride=-1024) == -6
 
 
 def test_decode_refuses_cpu_tensors():

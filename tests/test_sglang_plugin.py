@@ -251,3 +251,85 @@ def test_hook_matches_dense_attention(device, dtype):
     paths2 = [table[rows[r], : lens[r] + 1].cpu().long() for r in range(n)]
     want2 = oracle.dense_attention(q.view(n, hq, d).cpu(), k_pool.cpu(), v_pool.cpu(), paths2, layer.scaling)
     assert_parity(o2.view(n, hq, d).cpu(), want2, "hook after step", out_dtype=dtype)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("loc_dtype", [torch.int32, torch.int64])
+def test_store_kv_cache_equals_the_two_indexed_assignments(device, dtype, loc_dtype):
+    """One launch for both pools against torch's indexed assignment, bit for bit: flat and
+    three-dimensional new rows, rows that are a slice of a wider tensor (qkv projections), pools
+    with padded slot strides, int32 and int64 slots; slots outside the pool are skipped."""
+    from fasttree_hip.decode import store_kv_cache
+
+    g = torch.Generator().manual_seed(5)
+    hkv, d, slots, n = 8, 128, 500, 37
+    wide_k = torch.randn((slots, hkv + 2, d), generator=g).to(dtype).to(device)
+    k_pool, v_pool = wide_k[:, 1:-1], torch.randn((slots, hkv, d), generator=g).to(dtype).to(device)
+    qkv = torch.randn((n, 3 * hkv * d), generator=g).to(dtype).to(device)
+    k_new, v_new = qkv[:, hkv * d: 2 * hkv * d], qkv[:, 2 * hkv * d:]
+    loc = torch.randperm(slots, generator=g)[:n].to(loc_dtype).to(device)
+    want_k, want_v, want_wide = k_pool.clone(), v_pool.clone(), wide_k.clone()
+    want_k[loc.long()] = k_new.reshape(n, hkv, d)
+    want_v[loc.long()] = v_new.reshape(n, hkv, d)
+    store_kv_cache(k_new, v_new, loc, k_pool, v_pool)
+    torch.cuda.synchronize()
+    assert torch.equal(k_pool, want_k) and torch.equal(v_pool, want_v)
+    assert torch.equal(wide_k[:, 0], want_wide[:, 0]) and torch.equal(wide_k[:, -1], want_wide[:, -1])
+    # out of range: skipped, everything else written
+    loc2 = loc.clone()
+    loc2[3], loc2[11] = slots, -1
+    k_new2 = torch.randn((n, hkv, d), generator=g).to(dtype).to(device)
+    keep = torch.ones(n, dtype=torch.bool)
+    keep[3] = keep[11] = False
+    want_k[loc[keep.to(device)].long()] = k_new2[keep.to(device)]
+    want_v[loc[keep.to(device)].long()] = k_new2[keep.to(device)]
+    store_kv_cache(k_new2, k_new2.clone(), loc2, k_pool, v_pool)
+    torch.cuda.synchronize()
+    assert torch.equal(k_pool, want_k) and torch.equal(v_pool, want_v)
+    store_kv_cache(k_new2[:0], k_new2[:0], loc2[:0], k_pool, v_pool)  # no tokens: nothing to do
+    with pytest.raises(Exception):
+        store_kv_cache(k_new2.float(), k_new2.float(), loc2, k_pool, v_pool)
+    with pytest.raises(Exception):
+        store_kv_cache(k_new2, k_new2, loc2[:5], k_pool, v_pool)
+
+
+@pytest.mark.gpu
+def test_hook_with_the_fused_store(device):
+    """FastTreeMetadata(fused_store=True): the hook writes the new rows itself (the layer's
+    store_kv_cache is not called) and attends them."""
+    import fasttree_oracle as oracle
+    from helpers import assert_parity
+
+    rng = random.Random(9)
+    hq, hkv, d, dtype = 32, 8, 128, torch.float16
+    system = [rng.randint(1, 10**6) for _ in range(50)]
+    prompts = [system + [rng.randint(1, 10**6) for _ in range(rng.randint(1, 30))] for _ in range(12)]
+    outputs = [[rng.randint(1, 10**6) for _ in range(rng.randint(0, 4))] for _ in prompts]
+    n = len(prompts)
+    batch, n_slots = make_batch(prompts, outputs, [system], device=device, max_ctx=128)
+    meta = small_meta(device=device, fused_store=True)
+    prepare_for_fasttree_meta(batch, meta)
+    g = torch.Generator().manual_seed(4)
+    k_pool = torch.randn((n_slots + 8, hkv, d), generator=g).to(dtype).to(device)
+    v_pool = torch.randn((n_slots + 8, hkv, d), generator=g).to(dtype).to(device)
+    q = torch.randn((n, hq * d), generator=g).to(dtype).to(device)
+    k_new = torch.randn((n, hkv * d), generator=g).to(dtype).to(device)
+    v_new = torch.randn((n, hkv * d), generator=g).to(dtype).to(device)
+    table = batch.req_to_token_pool.req_to_token
+    lens = [len(p) + len(o) + 1 for p, o in zip(prompts, outputs)]
+    out_loc = torch.tensor([int(table[r, lens[r] - 1]) for r in range(n)], device=device, dtype=torch.int32)
+    im = Obj(token_to_kv_pool=FakePool(k_pool, v_pool), req_to_token_pool=batch.req_to_token_pool,
+             fasttree=meta, out_cache_loc=out_loc)
+    layer = FakeLayer(hq, hkv, d)
+
+    def refuse(*a, **k):
+        raise AssertionError("the layer's store_kv_cache must not be called")
+    layer.store_kv_cache = refuse
+    layer.decode_forward = decode_forward_fasttree.__get__(layer)
+    o = layer.decode_forward(q, k_new, v_new, im)
+    torch.cuda.synchronize()
+    assert torch.equal(k_pool[out_loc.long()], k_new.view(n, hkv, d)) and torch.equal(v_pool[out_loc.long()], v_new.view(n, hkv, d))
+    paths = [table[r, : lens[r]].cpu().long() for r in range(n)]
+    want = oracle.dense_attention(q.view(n, hq, d).cpu(), k_pool.cpu(), v_pool.cpu(), paths, layer.scaling)
+    assert_parity(o.view(n, hq, d).cpu(), want, "hook, fused store", out_dtype=dtype)
