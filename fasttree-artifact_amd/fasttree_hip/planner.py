@@ -430,8 +430,12 @@ LIGHT_VNODE_ROWS = 64
 WIDE_BLOCK_SLOTS = 512
 
 
+#: Query rows one block of the first-phase kernel serves per pass.
+WIDE_BLOCK_ROWS = 128
+
+
 def vnodes_in_launch_order(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, phase_node_offsets, group,
-                           num_kv_heads=None, light_work=None):
+                           num_kv_heads=None, light_work=None, q_tile=None):
     """The four per-vnode lists and the two phase lists, rearranged for the decode kernels.
 
     A vnode is the tuple (kv_offs[v], kv_lens[v], q_offs[v], q_lens[v]); nothing else refers to
@@ -455,8 +459,19 @@ def vnodes_in_launch_order(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, ph
       each to one wave that walks its run tile by tile: a long run that starts last is what the
       launch then waits for.
 
-    The order within the first phase is left alone (the kernel ranks those vnodes itself).
-    Returns ``(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, phase_node_offsets)``.
+    * with ``q_tile`` (the first phase's query tile, in requests) given: neighbours in the
+      first phase that attend the same KV run with adjoining scratch rows -- the query tiles one
+      node was cut into (fasttree.py:212-231) -- are joined into one vnode of at most
+      ``WIDE_BLOCK_ROWS x ceil(q_tile x group / WIDE_BLOCK_ROWS)`` query rows, what the blocks of
+      one vnode serve in a single pass: a tile of 16 requests x 4 heads fills half of a block's
+      rows, and two such tiles would stage the same run twice.  Not done while the first phase
+      has no more blocks than the machine has compute units (two half-filled blocks side by
+      side finish sooner than one full block).  The kernel joins such neighbours itself when
+      it is handed the reference's lists; joined here, no block is launched for the tiles
+      that were absorbed.
+
+    The order within the first phase is otherwise left alone (the kernel ranks those vnodes
+    itself).  Returns ``(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, phase_node_offsets)``.
     """
     light_work = LIGHT_VNODE_WORK if light_work is None else light_work
     lists = [np.array(x, dtype=np.int32, copy=True) for x in (kv_offs, kv_lens, q_offs, q_lens)]
@@ -474,7 +489,28 @@ def vnodes_in_launch_order(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, ph
     work = tokens[narrow] * ((rows[narrow] + 15) // 16)
     narrow = narrow[np.argsort(-work, kind="stable")]
     order = np.concatenate([wide, narrow])
-    return (*(x[order] for x in lists), [len(wide), len(narrow)], [0, len(wide)])
+    lists = [x[order] for x in lists]
+    n_wide = len(wide)
+    if q_tile is not None and n_wide > 1:
+        chunks = max(1, min(8, (int(q_tile) * int(group) + WIDE_BLOCK_ROWS - 1) // WIDE_BLOCK_ROWS))
+        heads = 1 if num_kv_heads is None else int(num_kv_heads)
+        if num_kv_heads is None or 2 * n_wide * heads * chunks > WIDE_BLOCK_SLOTS:
+            cap = WIDE_BLOCK_ROWS * chunks // int(group)  # requests
+            kept = [0]
+            kv_o, kv_l, q_o, q_l = (x[:n_wide].astype(np.int64) for x in lists)
+            q_l = q_l.copy()
+            for v in range(1, n_wide):
+                h = kept[-1]
+                if (kv_o[v] == kv_o[h] and kv_l[v] == kv_l[h] and q_o[h] + q_l[h] == q_o[v]
+                        and q_l[h] + q_l[v] <= cap):
+                    q_l[h] += q_l[v]
+                else:
+                    kept.append(v)
+            lists[3][:n_wide] = q_l.astype(np.int32)
+            keep = np.concatenate([np.array(kept, dtype=np.int64), np.arange(n_wide, len(order))])
+            lists = [x[keep] for x in lists]
+            n_wide = len(kept)
+    return (*lists, [n_wide, len(narrow)], [0, n_wide])
 
 
 def fasttree_preparation(
@@ -520,7 +556,8 @@ def fasttree_preparation(
     vnodes = (plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens,
               plan.phase_node_nums, plan.phase_node_offsets)
     if launch_order:
-        vnodes = vnodes_in_launch_order(*vnodes, max(1, num_qo_heads // num_kv_heads), num_kv_heads)
+        vnodes = vnodes_in_launch_order(*vnodes, max(1, num_qo_heads // num_kv_heads), num_kv_heads,
+                                        q_tile=params.TSQs[0])
     mid_o = torch.empty((rows, num_qo_heads, head_dim), dtype=torch.float32, device=device)
     mid_lse = torch.empty((rows, num_qo_heads), dtype=torch.float32, device=device)
     aux = (

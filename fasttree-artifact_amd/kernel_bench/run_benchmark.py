@@ -1,8 +1,11 @@
 """The reference's kernel sweep (kernel_bench/run_benchmark.sh:5-92) in one process, with the table
 its parse_output.py / plot_norm_perf.py derive: 15 level-regular trees x 3 head configurations;
-per case the gathered decode without sharing ("flash attn"), the tree decode, and the two
-ablations of the tree decode (gamma = 10 with one KV split: every request its own full path,
-"naive"; gamma = -10: never merge, "w/o greedy").
+per case the gathered decode without sharing ("flash attn"), the tree decode, the two ablations
+of the tree decode (gamma = 10 with one KV split: every request its own full path, "naive";
+gamma = -10: never merge, "w/o greedy"), and the never-merge plan without KV splits
+("node-wise": every tree node one batched attention over its own KV, merged per request -- the
+schedule of a multi-level cascade attention, which the reference measures with FlashInfer,
+kernel_bench/bench_cascade.py).
 
     python run_benchmark.py --out sweep --preset mi355x [--cases 0,8,9] [--heads "32 8"]
 
@@ -68,6 +71,8 @@ def run_case(out_dir, nodes, contexts, q_heads, k_heads, preset, log=print, extr
                           "--kv_split_sizes", "81920,81920", "--signature", "fasttree 10"]),
         ("no_greedy", base + ["--choice", "fasttree", "--alpha", "0", "--beta", "0", "--gamma", "-10",
                               "--kv_split_sizes", "1024,128", "--signature", "fasttree -10"]),
+        ("node_wise", base + ["--choice", "fasttree", "--alpha", "0", "--beta", "0", "--gamma", "-10",
+                              "--kv_split_sizes", "81920,81920", "--signature", "fasttree node-wise"]),
     ]
     row = {"tree": f"{nodes} / {contexts}", "heads": f"{q_heads}/{k_heads}", "preset": preset}
     with open(out_path, "w") as fh:
@@ -85,20 +90,20 @@ def run_case(out_dir, nodes, contexts, q_heads, k_heads, preset, log=print, extr
             else:
                 row[tag] = next(iter(v for k, v in res.items() if k.startswith("fasttree")), None)
     log(f"{row['tree']:60s} {row['heads']:6s} {preset:9s} gathered {row['flash_attn']:.4f} ms  tree {row['fasttree']:.4f} ms  "
-        f"naive {row['naive']:.4f}  w/o greedy {row['no_greedy']:.4f}  check {row['check']}  max abs {row['max_abs']:.1e}")
+        f"naive {row['naive']:.4f}  w/o greedy {row['no_greedy']:.4f}  node-wise {row['node_wise']:.4f}  check {row['check']}  max abs {row['max_abs']:.1e}")
     return row
 
 
 def write_table(rows, path):
-    engines = ["flash_attn", "naive", "no_greedy", "fasttree"]
+    engines = ["flash_attn", "naive", "node_wise", "no_greedy", "fasttree"]
     with open(path, "w") as fh:
-        fh.write("| tree (nodes / tokens per level) | q/kv heads | preset | gathered ms | tree, naive ms | tree, w/o greedy ms | tree ms | "
-                 "speed-up over gathered | normalised: gathered / naive / w/o greedy / tree | allclose 1e-2 | max abs | worst request mean abs |\n")
-        fh.write("|---|---|---|---|---|---|---|---|---|---|---|---|\n")
+        fh.write("| tree (nodes / tokens per level) | q/kv heads | preset | gathered ms | tree, naive ms | node-wise ms | tree, w/o greedy ms | tree ms | "
+                 "speed-up over gathered | normalised: gathered / naive / node-wise / w/o greedy / tree | allclose 1e-2 | max abs | worst request mean abs |\n")
+        fh.write("|---|---|---|---|---|---|---|---|---|---|---|---|---|\n")
         for r in rows:
             best = min(r[e] for e in engines)
             norm = " / ".join(f"{best / r[e]:.2f}" for e in engines)
-            fh.write(f"| {r['tree']} | {r['heads']} | {r['preset']} | {r['flash_attn']:.4f} | {r['naive']:.4f} | {r['no_greedy']:.4f} | "
+            fh.write(f"| {r['tree']} | {r['heads']} | {r['preset']} | {r['flash_attn']:.4f} | {r['naive']:.4f} | {r['node_wise']:.4f} | {r['no_greedy']:.4f} | "
                      f"{r['fasttree']:.4f} | {r['flash_attn'] / r['fasttree']:.2f} | {norm} | {'passed' if r['check'] else 'FAILED'} | "
                      f"{r['max_abs']:.1e} | {r['mean_abs']:.1e} |\n")
         fh.write("\n")

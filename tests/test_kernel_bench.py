@@ -56,12 +56,12 @@ def test_sweep_lists_and_table():
 
 
 def test_sweep_table_is_normalised_to_the_best_engine(tmp_path):
-    row = dict(tree="1,2 / 8,8", heads="32/8", preset="mi355x", flash_attn=0.4, naive=0.2, no_greedy=0.1, fasttree=0.05,
+    row = dict(tree="1,2 / 8,8", heads="32/8", preset="mi355x", flash_attn=0.4, naive=0.2, node_wise=0.2, no_greedy=0.1, fasttree=0.05,
                check=True, max_abs=1e-4, mean_abs=1e-5)
     path = tmp_path / "r.md"
     run_benchmark.write_table([row], str(path))
     body = path.read_text().split("\n")[2]
-    assert "| 8.00 |" in body and "0.12 / 0.25 / 0.50 / 1.00" in body and "passed" in body
+    assert "| 8.00 |" in body and "0.12 / 0.25 / 0.25 / 0.50 / 1.00" in body and "passed" in body
 
 
 @pytest.mark.gpu

@@ -164,6 +164,48 @@ def test_launch_order_is_a_permutation_of_the_vnodes(name, light_work):
     assert nums_few == (nums if wide > 512 else list(plan.phase_node_nums))
 
 
+@pytest.mark.parametrize("name", ["c3", "c5_seed0", "shape07_h32_8", "rand17", "rand41"])
+def test_launch_order_joins_query_tiles_without_changing_what_is_computed(name):
+    """With the query tile given, neighbouring tiles of one run become one vnode of at most 128
+    rows x chunks: every (run, scratch row) pair is still served exactly once."""
+    from fasttree_hip.planner import vnodes_in_launch_order
+    case = next(c for c in PLANNER_CASES if c["name"] == name)
+    tree, ptrs, batch, plan, params, _ = run_planner(case)
+    group = case["Hq"] // case["Hkv"]
+
+    def pairs(kv_offs, kv_lens, q_offs, q_lens):
+        out = []
+        for ko, kl, qo, ql in zip(kv_offs, kv_lens, q_offs, q_lens):
+            out.extend((int(ko), int(kl), int(qo) + i) for i in range(int(ql)))
+        return sorted(out)
+
+    before = pairs(plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens)
+    q_tile = plan.q_tile_sizes[0]
+    *lists, nums, offs = vnodes_in_launch_order(
+        plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens,
+        plan.phase_node_nums, plan.phase_node_offsets, group, None, light_work=0, q_tile=q_tile)
+    assert pairs(*lists) == before
+    assert len(set(p[2] for p in before)) == plan.num_rows == len(before)
+    chunks = max(1, min(8, -(-q_tile * group // 128)))
+    cap = 128 * chunks // group
+    wide_q = lists[3][:nums[0]]
+    assert nums[1] == plan.phase_node_nums[1] and nums[0] <= plan.phase_node_nums[0] and offs == [0, nums[0]]
+    assert all(q <= max(cap, q_tile) for q in wide_q)
+    # no two neighbours left that could still be joined
+    for v in range(1, nums[0]):
+        same = lists[0][v] == lists[0][v - 1] and lists[1][v] == lists[1][v - 1] and lists[2][v - 1] + lists[3][v - 1] == lists[2][v]
+        assert not (same and lists[3][v - 1] + lists[3][v] <= cap)
+    if name == "c3":
+        # 100 root tiles of 16 requests in 4 splits -> 13 per split; 10 x (16, 16, 8) -> 10 x (32, 8)
+        assert plan.phase_node_nums[0] == 130 and nums[0] == 4 * 13 + 10 * 2
+    # with the kv heads given and no more blocks than compute units, nothing is joined
+    *_, nums_few, _ = vnodes_in_launch_order(
+        plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens,
+        plan.phase_node_nums, plan.phase_node_offsets, group, 1, light_work=0, q_tile=q_tile)
+    if 2 * plan.phase_node_nums[0] * chunks <= 512:
+        assert nums_few == list(plan.phase_node_nums)
+
+
 def test_ablation_extremes():
     """gamma = +10 with alpha = beta = 0 merges every node into its leaf path (one vnode per
     request over its whole path); gamma = -10 never merges."""
