@@ -439,3 +439,42 @@ def test_narrow_vnode_wider_than_its_tile_argument_with_shared_waves(device):
     aux[11], aux[12] = [0, sum(aux[11])], [0, 0]
     o = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, [4, 4], [32, 32], 1.0 / math.sqrt(128))
     _dense_check(tree, inp, o, "narrow passes")
+
+
+@pytest.mark.gpu
+def test_decode_replays_from_a_captured_graph(device):
+    """The decode call allocates nothing and only enqueues launches on the stream it is given, so
+    a caller can capture it: the graph is replayed several times, with eager work, new inputs
+    and synchronisations in between, and every replay is compared with the eager result."""
+    _announce("graph capture")
+    tree, ptrs, batch = build_tree({"kind": "regular", "sizes": [1, 6, 48], "lens": [700, 90, 21]})
+    inp = make_decode_inputs(tree, 32, 8, 128, device=device, dtype=torch.float16, seed=5, shuffle_slots=True)
+    params = FastTreeParams()
+    params.set_values(0.66, 0.33, 0.1); params.set_q_tile_sizes([16, 4]); params.set_kv_tile_sizes([32, 32])
+    params.set_kv_group_num(4)
+    aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, 32, 8, 128, [1024, 128], [132, 528], [132, 132], params,
+                                  device=device, kv_slot_map=inp.slot_map)
+    scale = 1.0 / math.sqrt(128)
+    q = inp.Q.clone()
+    o_graph = torch.empty_like(q)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fasttree_decode(q, inp.K_pool, inp.V_pool, o_graph, *aux, [16, 4], [32, 32], scale)  # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        fasttree_decode(q, inp.K_pool, inp.V_pool, o_graph, *aux, [16, 4], [32, 32], scale)
+    gen = torch.Generator().manual_seed(1)
+    for replay in range(4):
+        q.copy_(torch.randn(q.shape, generator=gen).to(q.dtype))  # new queries in the captured buffer
+        o_graph.fill_(float("nan"))
+        aux[9].fill_(float("nan")); aux[10].fill_(float("nan"))     # the scratch is rewritten by every replay
+        graph.replay()
+        torch.cuda.synchronize()
+        o_eager = torch.empty_like(q)
+        fasttree_decode(q, inp.K_pool, inp.V_pool, o_eager, *aux, [16, 4], [32, 32], scale)
+        torch.cuda.synchronize()
+        assert torch.equal(o_graph, o_eager), f"replay {replay}"
+    inp.Q.copy_(q)
+    _dense_check(tree, inp, o_graph, "graph replay")
