@@ -435,7 +435,7 @@ WIDE_BLOCK_ROWS = 128
 
 
 def vnodes_in_launch_order(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, phase_node_offsets, group,
-                           num_kv_heads=None, light_work=None, q_tile=None):
+                           num_kv_heads=None, light_work=None, q_tile=None, return_order=False):
     """The four per-vnode lists and the two phase lists, rearranged for the decode kernels.
 
     A vnode is the tuple (kv_offs[v], kv_lens[v], q_offs[v], q_lens[v]); nothing else refers to
@@ -471,7 +471,9 @@ def vnodes_in_launch_order(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, ph
       that were absorbed.
 
     The order within the first phase is otherwise left alone (the kernel ranks those vnodes
-    itself).  Returns ``(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, phase_node_offsets)``.
+    itself).  Returns ``(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, phase_node_offsets)``;
+    with ``return_order`` a seventh element: for every vnode of the input its position in the
+    output, or -1 for a query tile that was absorbed into its neighbour.
     """
     light_work = LIGHT_VNODE_WORK if light_work is None else light_work
     lists = [np.array(x, dtype=np.int32, copy=True) for x in (kv_offs, kv_lens, q_offs, q_lens)]
@@ -491,6 +493,7 @@ def vnodes_in_launch_order(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, ph
     order = np.concatenate([wide, narrow])
     lists = [x[order] for x in lists]
     n_wide = len(wide)
+    kept_all = np.arange(len(order))
     if q_tile is not None and n_wide > 1:
         chunks = max(1, min(8, (int(q_tile) * int(group) + WIDE_BLOCK_ROWS - 1) // WIDE_BLOCK_ROWS))
         heads = 1 if num_kv_heads is None else int(num_kv_heads)
@@ -510,7 +513,13 @@ def vnodes_in_launch_order(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, ph
             keep = np.concatenate([np.array(kept, dtype=np.int64), np.arange(n_wide, len(order))])
             lists = [x[keep] for x in lists]
             n_wide = len(kept)
-    return (*lists, [n_wide, len(narrow)], [0, n_wide])
+            kept_all = keep
+    result = (*lists, [n_wide, len(narrow)], [0, n_wide])
+    if return_order:
+        where = np.full(len(order), -1, dtype=np.int64)
+        where[order[kept_all]] = np.arange(len(kept_all))
+        result = (*result, where)
+    return result
 
 
 def fasttree_preparation(

@@ -51,6 +51,7 @@ class FastTreeMetadata:
         max_vnode_to_q_entries: int = 81920,
         max_batch_size: int = 8192,
         fused_store: bool = False,
+        launch_order: bool = True,
     ):
         self.num_qo_heads = num_qo_heads
         self.num_kv_heads = num_kv_heads
@@ -66,6 +67,9 @@ class FastTreeMetadata:
         #: not in the reference: the hook writes the step's K/V rows with this library's single
         #: launch instead of calling the layer's ``store_kv_cache``
         self.fused_store = fused_store
+        #: not in the reference: the vnode lists are arranged for the kernels
+        #: (planner.vnodes_in_launch_order) instead of left in the reference's order
+        self.launch_order = launch_order
 
         def ints(n):
             return torch.empty(n, dtype=torch.int32, device=device)
@@ -267,16 +271,27 @@ def prepare_for_fasttree_meta(batch, fasttree_metadata: FastTreeMetadata):
     perm = above + below
     meta.phase_node_nums = [len(above), len(below)]
     meta.phase_node_offsets = [0, len(above)]
+    lists = [[x[i] for i in perm] for x in (kv_offs, kv_lens, q_offs, q_lens)]
+    if getattr(meta, "launch_order", False):
+        from .planner import vnodes_in_launch_order
+
+        *arranged, nums, offs, where = vnodes_in_launch_order(
+            *lists, meta.phase_node_nums, meta.phase_node_offsets, meta.kv_group_num, meta.num_kv_heads,
+            q_tile=q_tiles[0], return_order=True)
+        lists = [x.tolist() for x in arranged]
+        meta.phase_node_nums, meta.phase_node_offsets = nums, offs
+        # (the tail vnodes are single-request vnodes of the second phase: never absorbed)
+        meta.req_last_vnodes = [int(where[v]) for v in meta.req_last_vnodes]
 
     def upload(dst, values):
         src = torch.tensor(values, device="cpu", dtype=torch.int32)
         dst[: src.numel()].copy_(src, non_blocking=True)
 
     upload(meta.vnode_to_q_entries, q_entries)
-    upload(meta.vnode_to_q_offs, [q_offs[i] for i in perm])
-    upload(meta.vnode_to_q_lens, [q_lens[i] for i in perm])
-    upload(meta.vnode_to_kv_offs, [kv_offs[i] for i in perm])
-    upload(meta.vnode_to_kv_lens, [kv_lens[i] for i in perm])
+    upload(meta.vnode_to_kv_offs, lists[0])
+    upload(meta.vnode_to_kv_lens, lists[1])
+    upload(meta.vnode_to_q_offs, lists[2])
+    upload(meta.vnode_to_q_lens, lists[3])
     upload(meta.req_to_vnode_entries, req_entries)
     upload(meta.req_to_vnode_offs, req_offs)
     upload(meta.req_to_vnode_lens, req_lens)

@@ -112,7 +112,7 @@ def test_hand_derived_plan():
     prompts = [[1, 2, 3, 4, 5, 6], [1, 2, 3, 4, 7, 8, 9], [1, 2, 3, 4, 7, 8, 9]]
     outputs = [[10, 11], [12], []]
     batch, _ = make_batch(prompts, outputs, shared_prefixes=[[1, 2, 3, 4]], row_of=[2, 0, 5])
-    meta = small_meta()
+    meta = small_meta(launch_order=False)  # the reference's own order
     prepare_for_fasttree_meta(batch, meta)
     s = 64  # row stride of req_to_token
     # parallelism [0, 24] < thresholds: pass 0 leaves the splits, pass 1 takes its second branch
@@ -130,6 +130,21 @@ def test_hand_derived_plan():
     assert batch.fasttree_metadata is meta
     prepare_for_fasttree_step(batch, meta)
     assert meta.vnode_to_kv_lens[:6].tolist() == [4, 2, 3, 4, 3, 2]
+
+    # launch order (the default): the same vnodes, longest first within the phase; the tail
+    # vnodes are found at their new positions
+    meta2 = small_meta()
+    prepare_for_fasttree_meta(batch, meta2)
+    got2 = plan_lists(meta2, batch)
+    vnodes = lambda g: sorted(zip(g["kv_offs"], g["kv_lens"], g["q_offs"], g["q_lens"]))
+    assert vnodes(got2) == vnodes(got) and list(meta2.phase_node_nums) == [0, 6]
+    assert got2["kv_lens"] == [4, 3, 3, 2, 2, 1]
+    for key in ("q_entries", "req_entries", "req_offs", "req_lens"):
+        assert got2[key] == got[key]
+    for r, v in enumerate(meta2.req_last_vnodes):
+        assert (got2["kv_offs"][v], got2["q_offs"][v]) == (got["kv_offs"][[3, 4, 5][r]], got["q_offs"][[3, 4, 5][r]])
+    prepare_for_fasttree_step(batch, meta2)
+    assert sorted(meta2.vnode_to_kv_lens[:6].tolist()) == sorted([4, 2, 3, 4, 3, 2])
 
 
 def covered_slots(meta, batch):
