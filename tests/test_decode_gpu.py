@@ -412,6 +412,22 @@ def test_more_wide_vnodes_than_the_ranking_holds(device):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("d", [64, 128, 256])
+def test_light_wide_vnodes_run_with_the_narrow_phase_at_every_head_size(d, device):
+    """More first-phase blocks than the device holds, all of them light (32-64 rows x 20-30
+    tokens): the launch order hands them to the narrow path, which serves them in passes of 16
+    rows (head_dim 256 goes through the register-staged kernel)."""
+    _announce("light wide vnodes", d)
+    aux = _plan_and_check(device, [1, 150, 1200], [20, 30, 9], 16, 4, d, [16, 4], [1024, 128], f"light wide d{d}",
+                          sample=list(range(0, 1200, 23)), thr=((132, 528), (132, 132)))
+    wide = aux[11][0]
+    assert wide == 0 and int(aux[5].max()) * 4 > 16, "every vnode is launched narrow, some with more than 16 rows"
+    aux = _plan_and_check(device, [1, 150, 1200], [20, 30, 9], 16, 4, d, [16, 4], [1024, 128], f"light wide d{d}, planner order",
+                          sample=list(range(0, 1200, 23)), thr=((132, 528), (132, 132)), launch_order=False)
+    assert aux[11][0] == 225
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("batch", [1, 5, 40, 150])
 def test_few_long_narrow_vnodes_are_shared_between_waves(batch, device):
     """Few requests with long private runs: 8, 4 or 2 waves share a narrow vnode (all-narrow
