@@ -49,13 +49,13 @@ def random_case(seed):
                 launch_order=rng.random() < 0.7)
 
 
-@pytest.mark.parametrize("seed", list(range(48)))
+# (seeds 24 and 44 draw pools of more than 2**27 elements and are left out)
+@pytest.mark.parametrize("seed", [s for s in range(50) if s not in (24, 44)])
 def test_random_tree_and_settings(seed, device):
     c = random_case(seed)
     print("\n[gpu case] random", seed, {k: v for k, v in c.items() if k != "spec"}, c["spec"], flush=True)
     tree, ptrs, batch = build_tree(c["spec"])
-    if ptrs[-1] * c["hkv"] * c["d"] > (1 << 27):
-        pytest.skip("pool larger than this test is meant for")
+    assert ptrs[-1] * c["hkv"] * c["d"] <= (1 << 27), "pool larger than this test is meant for"
     inp = make_decode_inputs(tree, c["hq"], c["hkv"], c["d"], device=device, dtype=c["dtype"], seed=seed, shuffle_slots=True)
     params = FastTreeParams()
     params.set_values(*c["abg"]); params.set_q_tile_sizes(list(c["q_tiles"])); params.set_kv_tile_sizes([32, 32])
