@@ -496,8 +496,9 @@ __global__ void __launch_bounds__(kBlock) stage1_kernel(Stage1Args a) {
 // ---------------------------------------------------------------------------------------
 // Wide vnodes: 32x32x16 MFMA tiles (twice the rate of 16x16x32 on this part), four waves per
 // block with 32 query rows each and two blocks per compute unit, so that two waves share a SIMD
-// and one wave's waits are filled by the other's instructions.  (Matrix and vector arithmetic
-// of the two do not run at the same time on this part: a tile step costs the sum of both.)
+// and one wave's waits are filled by the other's instructions.  (Within a wave a tile step is one
+// dependent chain, scores -> soft-max -> P.V; the matrix instructions of one wave overlap the
+// vector instructions of the other about half of the time.)
 // ---------------------------------------------------------------------------------------
 #ifdef FT_TIMING
 // Development aid, compiled out of the product: per-wave cycle counts of the wide kernel's
