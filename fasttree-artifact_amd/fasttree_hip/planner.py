@@ -425,7 +425,7 @@ def fasttree_plan(
 #: KV tokens is launched with the second phase when the first phase alone has more blocks than
 #: WIDE_BLOCK_SLOTS, the number an MI355X runs at a time (256 compute units x 2); see
 #: :func:`vnodes_in_launch_order`.
-LIGHT_VNODE_WORK = int(os.environ.get("FASTTREE_LIGHT_VNODE_WORK", "4096"))
+LIGHT_VNODE_WORK = 4096
 LIGHT_VNODE_ROWS = 64
 WIDE_BLOCK_SLOTS = 512
 
