@@ -494,3 +494,33 @@ def test_decode_replays_from_a_captured_graph(device):
         assert torch.equal(o_graph, o_eager), f"replay {replay}"
     inp.Q.copy_(q)
     _dense_check(tree, inp, o_graph, "graph replay")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_large_and_growing_scores(dtype, device):
+    """Scores of large magnitude that keep growing along every run (keys scaled by a ramp over
+    the token position, queries by 3): the running soft-max reference moves on almost every
+    tile, in the wide path, the narrow path and the shared-wave narrow path, and nothing
+    overflows.  (A near one-hot soft-max amplifies the fp32-vs-fp64 score difference, so the
+    bound here is the reference bench's 1e-2, not the parity bar.)"""
+    _announce("growing scores", dtype)
+    for sizes, lens, hq, hkv in (([1, 6, 60], [900, 130, 70], 32, 8), ([1, 3], [64, 1100], 16, 1)):
+        tree, ptrs, batch = build_tree({"kind": "regular", "sizes": sizes, "lens": lens})
+        inp = make_decode_inputs(tree, hq, hkv, 128, device=device, dtype=dtype, seed=21, shuffle_slots=False)
+        ramp = torch.linspace(1.0, 7.0, inp.K_pool.shape[0], device=device).view(-1, 1, 1)
+        inp.K_pool.copy_((inp.K_pool.float() * ramp).to(dtype))
+        inp.Q.copy_((inp.Q.float() * 3).to(dtype))
+        params = FastTreeParams()
+        g = hq // hkv
+        params.set_values(0.66, 0.33, 0.1); params.set_q_tile_sizes([max(1, 64 // g), max(1, 16 // g)])
+        params.set_kv_tile_sizes([32, 32]); params.set_kv_group_num(g)
+        aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, hq, hkv, 128, [1024, 128], [256, 1024], [256, 256], params,
+                                      device=device, kv_slot_map=inp.slot_map)
+        o = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, list(params.TSQs), [32, 32], 1.0 / math.sqrt(128))
+        assert torch.isfinite(o.float()).all()
+        paths = [inp.path_tokens[r] for r in range(batch)]
+        dense = oracle.dense_attention(inp.Q.cpu(), inp.K_pool.cpu(), inp.V_pool.cpu(), paths, 1.0 / math.sqrt(128))
+        err = (o.float().cpu() - dense.float()).abs().max().item()
+        print(f"growing scores {sizes} {dtype}: max abs {err:.2e}", flush=True)
+        assert err <= (1e-2 if dtype == torch.float16 else 4e-2)
