@@ -442,7 +442,7 @@ def vnodes_in_launch_order(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, ph
     a vnode by its position (the per-request lists of kernel_bench/fasttree.py:233-244 name
     scratch rows, not vnodes), and the kernels compute a vnode of any number of query rows in
     either phase, so the order within a phase and the phase a vnode is launched with change the
-    schedule, not the result.  Two changes against the reference's order (fasttree.py:246-259):
+    schedule, not the result.  Three changes against the reference's order (fasttree.py:246-259):
 
     * light first-phase vnodes -- at most :data:`LIGHT_VNODE_ROWS` query rows and query rows x
       KV tokens at most ``light_work`` (default :data:`LIGHT_VNODE_WORK`) -- move to the second
@@ -458,7 +458,6 @@ def vnodes_in_launch_order(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, ph
       equal work keeps the order).  The kernel hands these vnodes to the machine in list order,
       each to one wave that walks its run tile by tile: a long run that starts last is what the
       launch then waits for.
-
     * with ``q_tile`` (the first phase's query tile, in requests) given: neighbours in the
       first phase that attend the same KV run with adjoining scratch rows -- the query tiles one
       node was cut into (fasttree.py:212-231) -- are joined into one vnode of at most
