@@ -521,6 +521,47 @@ def vnodes_in_launch_order(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, ph
     return result
 
 
+class PlanBuffers:
+    """Device buffers for :func:`fasttree_preparation`, allocated once at stated maxima and
+    filled in place by every call that is given them: a serving loop re-plans whenever its batch
+    changes, and neither the nine index arrays nor the fp32 scratch should be allocated anew each
+    time (the reference says so of its own bench code, kernel_bench/fasttree.py:264, and
+    pre-allocates in its plugin, metadata.py:40-58).
+
+    ``max_kv_entries`` bounds the flat KV index list (unique tokens plus what merged chains
+    replicate, plus the 32 padding entries), ``max_rows`` the scratch rows (one per request and
+    KV split), ``max_vnodes`` the vnodes, ``max_batch_size`` the requests.
+    """
+
+    def __init__(self, num_qo_heads, head_dim, max_kv_entries, max_rows, max_vnodes, max_batch_size, device="cuda"):
+        import torch
+
+        def ints(n):
+            return torch.empty(int(n), dtype=torch.int32, device=device)
+
+        self.device = device
+        self.vnode_to_kv_entries = ints(max_kv_entries)
+        self.vnode_to_kv_offs, self.vnode_to_kv_lens = ints(max_vnodes), ints(max_vnodes)
+        self.vnode_to_q_entries = ints(max_rows)
+        self.vnode_to_q_offs, self.vnode_to_q_lens = ints(max_vnodes), ints(max_vnodes)
+        self.req_to_vnode_entries = ints(max_rows + 32)
+        self.req_to_vnode_offs, self.req_to_vnode_lens = ints(max_batch_size), ints(max_batch_size)
+        self.mid_o = torch.empty((int(max_rows), num_qo_heads, head_dim), dtype=torch.float32, device=device)
+        self.mid_lse = torch.empty((int(max_rows), num_qo_heads), dtype=torch.float32, device=device)
+
+    def fill(self, name, values):
+        """Copies ``values`` into the front of buffer ``name`` and returns that part of it."""
+        import torch
+
+        host = torch.from_numpy(np.ascontiguousarray(np.asarray(values, dtype=np.int32)))
+        dst = getattr(self, name)
+        if host.numel() > dst.numel():
+            raise ValueError(f"{name}: {host.numel()} entries do not fit the {dst.numel()} that were allocated")
+        part = dst[: host.numel()]
+        part.copy_(host)
+        return part
+
+
 def fasttree_preparation(
     tree_info,
     KV_ptrs,
@@ -536,6 +577,7 @@ def fasttree_preparation(
     device="cuda",
     kv_slot_map=None,
     launch_order=True,
+    buffers=None,
 ):
     """Drop-in for kernel_bench/fasttree.py:99-296: plan on the host, then place the nine
     int32 index arrays and the two fp32 partial-result buffers on ``device``.
@@ -547,7 +589,8 @@ def fasttree_preparation(
     in the reference: ``device`` defaults to the reference's hard-wired "cuda";
     ``kv_slot_map`` is described in :func:`fasttree_plan`; ``launch_order`` arranges the vnodes
     for the kernels (:func:`vnodes_in_launch_order`) instead of leaving them in the reference's
-    order.
+    order; with ``buffers`` (a :class:`PlanBuffers`) nothing is allocated on the device: the
+    arrays are written into its buffers and the returned tensors are their leading parts.
     """
     import torch
 
@@ -556,7 +599,13 @@ def fasttree_preparation(
         KV_SPLIT_SIZES, para_threshs1, para_threshs2, params, kv_slot_map=kv_slot_map,
     )
 
+    names = iter(("vnode_to_kv_entries", "vnode_to_kv_offs", "vnode_to_kv_lens", "vnode_to_q_entries", "vnode_to_q_offs",
+                  "vnode_to_q_lens", "req_to_vnode_entries", "req_to_vnode_offs", "req_to_vnode_lens"))
+
     def put(values):
+        name = next(names)  # (the nine arrays are placed in this order below)
+        if buffers is not None:
+            return buffers.fill(name, values)
         host = torch.from_numpy(np.ascontiguousarray(np.asarray(values, dtype=np.int32)))
         return host.to(device)
 
@@ -566,8 +615,14 @@ def fasttree_preparation(
     if launch_order:
         vnodes = vnodes_in_launch_order(*vnodes, max(1, num_qo_heads // num_kv_heads), num_kv_heads,
                                         q_tile=params.TSQs[0])
-    mid_o = torch.empty((rows, num_qo_heads, head_dim), dtype=torch.float32, device=device)
-    mid_lse = torch.empty((rows, num_qo_heads), dtype=torch.float32, device=device)
+    if buffers is not None:
+        if rows > buffers.mid_o.shape[0] or buffers.mid_o.shape[1:] != (num_qo_heads, head_dim):
+            raise ValueError(f"the scratch of the buffers ({tuple(buffers.mid_o.shape)}) does not hold "
+                             f"{rows} rows of {num_qo_heads} x {head_dim}")
+        mid_o, mid_lse = buffers.mid_o[:rows], buffers.mid_lse[:rows]
+    else:
+        mid_o = torch.empty((rows, num_qo_heads, head_dim), dtype=torch.float32, device=device)
+        mid_lse = torch.empty((rows, num_qo_heads), dtype=torch.float32, device=device)
     aux = (
         put(plan.vnode_to_kv_entries),
         put(vnodes[0]),

@@ -524,3 +524,27 @@ def test_large_and_growing_scores(dtype, device):
         err = (o.float().cpu() - dense.float()).abs().max().item()
         print(f"growing scores {sizes} {dtype}: max abs {err:.2e}", flush=True)
         assert err <= (1e-2 if dtype == torch.float16 else 4e-2)
+
+
+@pytest.mark.gpu
+def test_plans_in_preallocated_buffers(device):
+    """Two different batches planned one after the other into the same PlanBuffers (the second
+    smaller than the first): the decode reads the leading parts of the buffers."""
+    from fasttree_hip.planner import PlanBuffers
+    _announce("plan buffers")
+    buffers = PlanBuffers(32, 128, max_kv_entries=60000, max_rows=8192, max_vnodes=4096, max_batch_size=1024, device=device)
+    first_ptrs = None
+    for sizes, lens in (([1, 10, 200], [1500, 300, 40]), ([1, 7], [700, 90])):
+        tree, ptrs, batch = build_tree({"kind": "regular", "sizes": sizes, "lens": lens})
+        inp = make_decode_inputs(tree, 32, 8, 128, device=device, dtype=torch.float16, seed=13, shuffle_slots=True)
+        params = FastTreeParams()
+        params.set_values(0.66, 0.33, 0.1); params.set_q_tile_sizes([16, 4]); params.set_kv_tile_sizes([32, 32])
+        params.set_kv_group_num(4)
+        buffers.mid_o.fill_(float("nan")); buffers.mid_lse.fill_(float("nan"))
+        aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, 32, 8, 128, [1024, 128], [256, 1024], [256, 256], params,
+                                      device=device, kv_slot_map=inp.slot_map, buffers=buffers)
+        now = [t.data_ptr() for t in aux[:11]]
+        assert first_ptrs is None or now == first_ptrs
+        first_ptrs = now
+        o = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, [16, 4], [32, 32], 1.0 / math.sqrt(128))
+        _dense_check(tree, inp, o, f"plan buffers {sizes}", list(range(0, batch, 3)))

@@ -206,6 +206,46 @@ def test_launch_order_joins_query_tiles_without_changing_what_is_computed(name):
         assert nums_few == list(plan.phase_node_nums)
 
 
+def test_preparation_into_preallocated_buffers():
+    """fasttree_preparation(buffers=...) writes into the same device buffers on every call and
+    returns their leading parts; the contents equal those of the allocating call."""
+    import torch
+    from fasttree_hip.planner import FastTreeParams, PlanBuffers, fasttree_preparation
+    buffers = PlanBuffers(32, 128, max_kv_entries=400000, max_rows=8192, max_vnodes=8192, max_batch_size=2048, device="cpu")
+    ptrs_seen = None
+    for name in ("c3", "c1", "shape07_h32_8"):
+        case = next(c for c in PLANNER_CASES if c["name"] == name)
+        tree, ptrs, batch = build_tree(case["tree"])
+        outs = []
+        for buf in (None, buffers):
+            params = FastTreeParams()
+            params.set_values(case["alpha"], case["beta"], case["gamma"]); params.set_q_tile_sizes(list(case["TSQs"]))
+            params.set_kv_tile_sizes(list(case["TSKs"])); params.set_kv_group_num(case["Hq"] // case["Hkv"])
+            if case["Hq"] != 32:
+                continue
+            outs.append(fasttree_preparation(tree, ptrs, batch, case["Hq"], case["Hkv"], 128, list(case["kv_split_sizes"]),
+                                             list(case["para_threshs1"]), list(case["para_threshs2"]), params,
+                                             device="cpu", buffers=buf))
+        if len(outs) < 2:
+            continue
+        (a, assign_a), (b, assign_b) = outs
+        assert assign_a == assign_b and a[11] == b[11] and a[12] == b[12]
+        for i in range(9):
+            assert torch.equal(a[i], b[i]), i
+        assert b[9].shape == a[9].shape and b[10].shape == a[10].shape
+        now = [t.data_ptr() for t in b[:11]]
+        assert ptrs_seen is None or now == ptrs_seen, "every call writes into the same buffers"
+        ptrs_seen = now
+    assert ptrs_seen is not None
+    small = PlanBuffers(32, 128, max_kv_entries=100, max_rows=4096, max_vnodes=2048, max_batch_size=512, device="cpu")
+    case = next(c for c in PLANNER_CASES if c["name"] == "c3")
+    tree, ptrs, batch = build_tree(case["tree"])
+    params = FastTreeParams()
+    params.set_values(0.66, 0.33, 0.1); params.set_q_tile_sizes([16, 4]); params.set_kv_tile_sizes([32, 32]); params.set_kv_group_num(4)
+    with pytest.raises(ValueError):
+        fasttree_preparation(tree, ptrs, batch, 32, 8, 128, [1024, 128], [132, 528], [132, 132], params, device="cpu", buffers=small)
+
+
 def test_ablation_extremes():
     """gamma = +10 with alpha = beta = 0 merges every node into its leaf path (one vnode per
     request over its whole path); gamma = -10 never merges."""
