@@ -310,6 +310,28 @@ def prepare_for_fasttree_step(batch, fasttree_metadata: FastTreeMetadata):
 # ---------------------------------------------------------------------------------------
 # Loader
 # ---------------------------------------------------------------------------------------
+def annotate_function(owner, func_name):
+    """Replaces ``owner.func_name`` by a version that runs inside a named profiler range with a
+    device synchronisation on either side, so that a trace shows the step's host and device time
+    under that name (plugin.py:70-83; the reference uses the ``nvtx`` package, this uses the
+    ranges torch exposes, which are roctx ranges on ROCm)."""
+    original = getattr(owner, func_name)
+
+    def annotated(*args, **kwargs):
+        if torch.cuda.is_available():
+            torch.cuda.synchronize()
+        torch.cuda.nvtx.range_push(func_name)
+        try:
+            return original(*args, **kwargs)
+        finally:
+            if torch.cuda.is_available():
+                torch.cuda.synchronize()
+            torch.cuda.nvtx.range_pop()
+
+    annotated.__wrapped__ = original
+    setattr(owner, func_name, annotated)
+
+
 def load_fasttree_plugin(enable_fasttree=True, annotate_breakdown=False):
     """Installs the hook into SGLang v0.2.13 (plugin.py:234-238).
 
@@ -318,7 +340,9 @@ def load_fasttree_plugin(enable_fasttree=True, annotate_breakdown=False):
     Without it, the three patches are applied here: ``RadixAttention.decode_forward``,
     ``InputMetadata.from_schedule_batch`` (carries ``batch.fasttree_metadata``), and
     ``ModelTpServer`` (metadata creation; a fresh plan when the batch changed, the ``+1`` step
-    otherwise, before every decode forward).  Raises ImportError when sglang is not installed.
+    otherwise, before every decode forward).  ``annotate_breakdown`` wraps the prefill and decode
+    forwards and the two planner entry points in named profiler ranges (plugin.py:68-89).
+    Raises ImportError when sglang is not installed.
     """
     if not enable_fasttree and not annotate_breakdown:
         print("[Warning] FastTree plugin is not enabled")
@@ -344,6 +368,12 @@ def load_fasttree_plugin(enable_fasttree=True, annotate_breakdown=False):
     from sglang.srt.managers.tp_worker import ModelTpServer
     from sglang.srt.model_executor.forward_batch_info import InputMetadata
 
+    if annotate_breakdown:
+        annotate_function(ModelTpServer, "forward_prefill_batch")
+        annotate_function(ModelTpServer, "forward_decode_batch")
+        if enable_fasttree:
+            annotate_function(this, "prepare_for_fasttree_meta")
+            annotate_function(this, "prepare_for_fasttree_step")
     if not enable_fasttree:
         return
 
@@ -381,9 +411,9 @@ def load_fasttree_plugin(enable_fasttree=True, annotate_breakdown=False):
     def decode_batch_with_plan(self, batch):
         members = tuple(id(r) for r in batch.reqs)
         if self._fasttree_planned_for == members:
-            prepare_for_fasttree_step(batch, self.fasttree_metadata)
+            this.prepare_for_fasttree_step(batch, self.fasttree_metadata)
         else:
-            prepare_for_fasttree_meta(batch, self.fasttree_metadata)
+            this.prepare_for_fasttree_meta(batch, self.fasttree_metadata)
             self._fasttree_planned_for = members
         return decode_batch(self, batch)
 

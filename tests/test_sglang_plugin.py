@@ -187,6 +187,27 @@ def test_every_token_is_covered_once(seed):
         assert all(got["q_entries"][i] == r for i in rows) and rows == sorted(rows)
 
 
+def test_annotate_function_keeps_results_and_errors():
+    """The breakdown wrapper of load_fasttree_plugin(annotate_breakdown=True): same result, same
+    exception, the original reachable, the range closed either way."""
+    from fasttree_hip.sglang_plugin import annotate_function
+    calls = []
+
+    class Owner:
+        def work(self, x, y=1):
+            calls.append((x, y))
+            if x < 0:
+                raise ValueError("negative")
+            return x + y
+
+    annotate_function(Owner, "work")
+    o = Owner()
+    assert o.work(2, y=5) == 7 and calls == [(2, 5)]
+    with pytest.raises(ValueError):
+        o.work(-1)
+    assert Owner.work.__wrapped__(o, 3) == 4
+
+
 # ---- the hook body on the GPU
 class FakeLayer:
     def __init__(self, hq, hkv, d, layer_id=0):
