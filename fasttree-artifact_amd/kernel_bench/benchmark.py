@@ -99,6 +99,16 @@ def main(args):
             name = args.signature
         out = func()
         ms, _, _ = do_bench(func, quantiles=QUANTILES)
+        if args.profile:
+            # one more call between the profiler's start and stop marks, inside a named range
+            # (kernel_bench/benchmark.py:12-24,60-63 does this with cudaProfilerStart/Stop)
+            torch.cuda.synchronize()
+            torch.cuda.profiler.start()
+            torch.cuda.nvtx.range_push(name)
+            func()
+            torch.cuda.synchronize()
+            torch.cuda.nvtx.range_pop()
+            torch.cuda.profiler.stop()
         print(f"{name} time:", ms, flush=True)
         results[name] = ms
         return out
@@ -168,6 +178,7 @@ def build_parser():
     parser.add_argument("--head_dim", type=int, default=128)
     parser.add_argument("--signature", type=str, default=None)
     parser.add_argument("--choice", type=str, choices=["flash_attn", "fasttree", "all"], default="all")
+    parser.add_argument("--profile", action="store_true", default=False)
     parser.add_argument("--mi355x", action="store_true", default=False,
                         help="query tiles and parallelism thresholds for MI355X instead of the H100 defaults")
     parser.add_argument("--quiet", action="store_true", default=False, help="do not print the planner's lines")

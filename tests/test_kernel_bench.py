@@ -38,7 +38,7 @@ def test_benchmark_options_and_defaults_follow_the_reference():
     assert (args.alpha, args.beta, args.gamma) == (0.66, 0.33, 0.1)
     assert args.kv_tile_size_per_phase == "32,32" and args.kv_split_sizes == "1024,128"
     assert (args.num_qo_heads, args.num_kv_heads, args.head_dim) == (32, 32, 128)
-    assert args.choice == "all" and args.signature is None and args.fasttree_heuristic_path is None
+    assert args.choice == "all" and args.signature is None and args.fasttree_heuristic_path is None and args.profile is False
     assert args.q_tile_size_per_phase is None and args.para_threshs1 is None and args.para_threshs2 is None
     with pytest.raises(SystemExit):
         benchmark.build_parser().parse_args(["--load_file_path", "x.txt", "--choice", "DeFT"])
@@ -81,5 +81,5 @@ def test_benchmark_runs_both_engines_and_checks_them(tmp_path, capsys):
     assert plan_path.read_text().startswith("Node 0: parent -1, assignment 0\n")
     res = benchmark.main(benchmark.build_parser().parse_args(
         ["--load_file_path", str(path), "--choice", "fasttree", "--alpha", "0", "--beta", "0", "--gamma", "10",
-         "--kv_split_sizes", "81920,81920", "--signature", "fasttree 10", "--quiet"]))
+         "--kv_split_sizes", "81920,81920", "--signature", "fasttree 10", "--quiet", "--profile"]))
     assert list(res) == ["fasttree 10"]
