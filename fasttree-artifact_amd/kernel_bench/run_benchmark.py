@@ -9,7 +9,8 @@ kernel_bench/bench_cascade.py).
 
     python run_benchmark.py --out sweep --preset mi355x [--cases 0,8,9] [--heads "32 8"]
 
-Writes ``<out>/trees/*.txt``, ``<out>/outputs/*.txt`` (the lines benchmark.py prints) and
+Writes ``<out>/trees/*.txt``, ``<out>/outputs/*.txt`` (``outputs_<preset>`` with ``--preset both``;
+the lines benchmark.py prints, under the file names the reference's parse_output.py reads) and
 ``<out>/results.md``: milliseconds per engine, the speed-up of the tree decode over the gathered
 decode, and performance normalised to the best engine of the row
 (kernel_bench/plot_norm_perf.py:27).
@@ -53,12 +54,13 @@ def reference_q_tiles(group):
     return {1: "64,16", 4: "16,4", 16: "4,1"}.get(group, f"{max(1, 64 // group)},{max(1, 16 // group)}")
 
 
-def run_case(out_dir, nodes, contexts, q_heads, k_heads, preset, log=print, extra=()):
+def run_case(out_dir, nodes, contexts, q_heads, k_heads, preset, log=print, extra=(), outputs="outputs"):
     tree = f"nc_{nodes}_{contexts}.txt"
     tree_path = os.path.join(out_dir, "trees", tree)
     if not os.path.exists(tree_path):
         tree_generation.main(["-n", nodes, "-l", contexts, "-o", tree_path])
-    out_path = os.path.join(out_dir, "outputs", f"nc_{nodes}_{contexts}_qk_{q_heads}_{k_heads}_{preset}.txt")
+    # (the file name the reference's parse_output.py expects, kernel_bench/parse_output.py:93)
+    out_path = os.path.join(out_dir, outputs, f"nc_{nodes}_{contexts}_qk_{q_heads}_{k_heads}.txt")
     base = ["--load_file_path", tree_path, "--num_qo_heads", str(q_heads), "--num_kv_heads", str(k_heads)]
     if preset == "mi355x":
         base += ["--mi355x"]
@@ -124,18 +126,20 @@ def main(argv=None):
     ap.add_argument("--heads", default=None, help='one head configuration, e.g. "32 8" (default: all three)')
     ap.add_argument("--extra", default="", help="further benchmark.py options for every run, as one string")
     args = ap.parse_args(argv)
-    for sub in ("trees", "outputs"):
+    presets = ["reference", "mi355x"] if args.preset == "both" else [args.preset]
+    outputs = {p: "outputs" if len(presets) == 1 else f"outputs_{p}" for p in presets}
+    for sub in ["trees", *outputs.values()]:
         os.makedirs(os.path.join(args.out, sub), exist_ok=True)
     cases = range(len(NODES_CONTEXTS)) if args.cases is None else [int(x) for x in args.cases.split(",")]
     heads = QK_HEADS if args.heads is None else [tuple(int(x) for x in args.heads.split())]
-    presets = ["reference", "mi355x"] if args.preset == "both" else [args.preset]
     rows = []
     for c in cases:
         nodes, contexts = NODES_CONTEXTS[c]
         for q_heads, k_heads in heads:
             for preset in presets:
                 rows.append(run_case(args.out, nodes, contexts, q_heads, k_heads, preset,
-                                     log=lambda *a: print(*a, flush=True), extra=args.extra.split()))
+                                     log=lambda *a: print(*a, flush=True), extra=args.extra.split(),
+                                     outputs=outputs[preset]))
                 write_table(rows, os.path.join(args.out, "results.md"))
     failed = [r for r in rows if not r["check"]]
     print(f"{len(rows)} cases, {len(failed)} failed the allclose check", flush=True)
