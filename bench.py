@@ -50,8 +50,9 @@ WORKLOADS = {
 
 # Planner arguments.  "reference" = the values the reference bench passes
 # (kernel_bench/benchmark.py:246-254, run_benchmark.sh:46-53: query tiles (64 // g, 16 // g)).
-# "mi355x" = the same planner with a wide-phase query tile of 256 // g requests (256 query
-# rows, the eight waves of a block) and thresholds sized for 256 compute units.
+# "mi355x" = the same tiles with the parallelism thresholds sized for 256 compute units instead of
+# an H100's 132; "wide" = as "mi355x" with a first-phase query tile of 256 // g requests (kept for
+# comparison: slower than "mi355x" over the reference's sweep now that query tiles are joined).
 # HBM bytes per stage-1 launch (read + write) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
 # each scaled by what the same counter reads for a plain copy of known size (2.000 and 1.000); the
 # runs and their commands are summarised in profiles/stage1_fused_stage2_<workload>_<dtype>.txt.
