@@ -51,7 +51,9 @@ WORKLOADS = {
 # Planner arguments.  "reference" = the values the reference bench passes
 # (kernel_bench/benchmark.py:246-254, run_benchmark.sh:46-53: query tiles (64 // g, 16 // g)).
 # "mi355x" = the same tiles with the parallelism thresholds sized for 256 compute units instead of
-# an H100's 132; "wide" = as "mi355x" with a first-phase query tile of 256 // g requests (kept for
+# an H100's 132 and a KV split of 256 instead of 128 tokens for phases short of parallelism (half
+# the partial rows per request; the launches that take it are small and bound by their
+# partials); "wide" = as "mi355x" with a first-phase query tile of 256 // g requests (kept for
 # comparison: slower than "mi355x" over the reference's sweep now that query tiles are joined).
 # HBM bytes per stage-1 launch (read + write) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
 # each scaled by what the same counter reads for a plain copy of known size (2.000 and 1.000); the
@@ -60,8 +62,8 @@ MEASURED_TRAFFIC = {("c3", "mi355x", "stage1"): 161.0e6, ("c4", "mi355x", "stage
 
 PRESETS = {
     "reference": dict(q_tiles=None, kv_tiles=(32, 32), kv_splits=(1024, 128), thr1=(132, 528), thr2=(132, 132)),
-    "mi355x": dict(q_tiles=None, kv_tiles=(32, 32), kv_splits=(1024, 128), thr1=(256, 1024), thr2=(256, 256)),
-    "wide": dict(q_tiles="wide", kv_tiles=(32, 32), kv_splits=(1024, 128), thr1=(256, 1024), thr2=(256, 256)),
+    "mi355x": dict(q_tiles=None, kv_tiles=(32, 32), kv_splits=(1024, 256), thr1=(256, 1024), thr2=(256, 256)),
+    "wide": dict(q_tiles="wide", kv_tiles=(32, 32), kv_splits=(1024, 256), thr1=(256, 1024), thr2=(256, 256)),
 }
 
 

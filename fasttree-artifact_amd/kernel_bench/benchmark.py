@@ -14,10 +14,11 @@ have no counterpart here.
 Timing follows the method of ``triton.testing.do_bench`` as the reference calls it
 (kernel_bench/benchmark.py:35,59): per-call device events, a 256 MB buffer cleared before every
 call, a repetition count sized for about 100 ms, the median reported in milliseconds.
-``--mi355x`` replaces the H100 defaults of the query tiles (64,16, right for 32/32 heads only) and
-of the parallelism thresholds with the ones for MI355X: tiles of 64 // g and 16 // g requests, as
-the reference's sweep picks them per GQA ratio (kernel_bench/run_benchmark.sh:46-53), and
-thresholds for 256 compute units instead of 132; explicit options win over it.
+``--mi355x`` replaces the H100 defaults of the query tiles (64,16, right for 32/32 heads only), of
+the parallelism thresholds and of the KV split sizes with the ones for MI355X: tiles of 64 // g
+and 16 // g requests, as the reference's sweep picks them per GQA ratio
+(kernel_bench/run_benchmark.sh:46-53), thresholds for 256 compute units instead of 132, and KV
+splits of 1024,256 instead of 1024,128 tokens; explicit options win over it.
 """
 import argparse
 import os
@@ -70,14 +71,14 @@ def main(args):
     num_qo_heads, num_kv_heads, head_dim = args.num_qo_heads, args.num_kv_heads, args.head_dim
     group = num_qo_heads // num_kv_heads
     dtype = torch.float16
-    defaults = dict(q_tile_size_per_phase="64,16", para_threshs1="132,528", para_threshs2="132,132")
+    defaults = dict(q_tile_size_per_phase="64,16", kv_split_sizes="1024,128", para_threshs1="132,528", para_threshs2="132,132")
     if args.mi355x:
-        defaults = dict(q_tile_size_per_phase=f"{max(1, 64 // group)},{max(1, 16 // group)}",
+        defaults = dict(q_tile_size_per_phase=f"{max(1, 64 // group)},{max(1, 16 // group)}", kv_split_sizes="1024,256",
                         para_threshs1="256,1024", para_threshs2="256,256")
     ints = lambda text: list(map(int, text.split(",")))
     Q_TILE_SIZE_PER_PHASE = ints(args.q_tile_size_per_phase or defaults["q_tile_size_per_phase"])
     KV_TILE_SIZE_PER_PHASE = ints(args.kv_tile_size_per_phase)
-    KV_SPLIT_SIZES = ints(args.kv_split_sizes)
+    KV_SPLIT_SIZES = ints(args.kv_split_sizes or defaults["kv_split_sizes"])
     para_threshs1 = ints(args.para_threshs1 or defaults["para_threshs1"])
     para_threshs2 = ints(args.para_threshs2 or defaults["para_threshs2"])
 
@@ -169,7 +170,7 @@ def build_parser():
     parser.add_argument("--gamma", type=float, default=0.1)
     parser.add_argument("--q_tile_size_per_phase", type=str, default=None, help="default 64,16")
     parser.add_argument("--kv_tile_size_per_phase", type=str, default="32,32")
-    parser.add_argument("--kv_split_sizes", type=str, default="1024,128")
+    parser.add_argument("--kv_split_sizes", type=str, default=None, help="default 1024,128")
     parser.add_argument("--para_threshs1", type=str, default=None, help="default 132,528")
     parser.add_argument("--para_threshs2", type=str, default=None, help="default 132,132")
     parser.add_argument("--fasttree_heuristic_path", type=str, default=None)
@@ -180,7 +181,7 @@ def build_parser():
     parser.add_argument("--choice", type=str, choices=["flash_attn", "fasttree", "all"], default="all")
     parser.add_argument("--profile", action="store_true", default=False)
     parser.add_argument("--mi355x", action="store_true", default=False,
-                        help="query tiles and parallelism thresholds for MI355X instead of the H100 defaults")
+                        help="query tiles, parallelism thresholds and KV split sizes for MI355X instead of the H100 defaults")
     parser.add_argument("--quiet", action="store_true", default=False, help="do not print the planner's lines")
     return parser
 

@@ -72,7 +72,7 @@ def run_case(out_dir, nodes, contexts, q_heads, k_heads, preset, log=print, extr
         ("naive", base + ["--choice", "fasttree", "--alpha", "0", "--beta", "0", "--gamma", "10",
                           "--kv_split_sizes", "81920,81920", "--signature", "fasttree 10"]),
         ("no_greedy", base + ["--choice", "fasttree", "--alpha", "0", "--beta", "0", "--gamma", "-10",
-                              "--kv_split_sizes", "1024,128", "--signature", "fasttree -10"]),
+                              "--signature", "fasttree -10"]),
         ("node_wise", base + ["--choice", "fasttree", "--alpha", "0", "--beta", "0", "--gamma", "-10",
                               "--kv_split_sizes", "81920,81920", "--signature", "fasttree node-wise"]),
     ]

@@ -36,10 +36,11 @@ def test_benchmark_options_and_defaults_follow_the_reference():
     defaults are resolved in main() so that --mi355x can replace them."""
     args = benchmark.build_parser().parse_args(["--load_file_path", "x.txt"])
     assert (args.alpha, args.beta, args.gamma) == (0.66, 0.33, 0.1)
-    assert args.kv_tile_size_per_phase == "32,32" and args.kv_split_sizes == "1024,128"
+    assert args.kv_tile_size_per_phase == "32,32"
     assert (args.num_qo_heads, args.num_kv_heads, args.head_dim) == (32, 32, 128)
     assert args.choice == "all" and args.signature is None and args.fasttree_heuristic_path is None and args.profile is False
     assert args.q_tile_size_per_phase is None and args.para_threshs1 is None and args.para_threshs2 is None
+    assert args.kv_split_sizes is None
     with pytest.raises(SystemExit):
         benchmark.build_parser().parse_args(["--load_file_path", "x.txt", "--choice", "DeFT"])
     with pytest.raises(SystemExit):
