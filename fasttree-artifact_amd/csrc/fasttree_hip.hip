@@ -129,7 +129,7 @@ struct Stage1Args {
   const int32_t* q_lens;
   int vnode_begin, vnode_count;    // vnodes served by wide blocks (or the whole range for the per-wave-staging kernel)
   int narrow_begin, narrow_count;  // vnodes of at most 16 rows
-  int narrow_share;                // waves that share one narrow vnode: 1, 2, 4 or 8
+  int narrow_share;                // waves that share one narrow vnode: 1, 2 or 4
   int wide_rows;                   // query rows the planner's tile gives a wide vnode (host hint for wide_chunks)
   int wide_chunks;                 // blocks per (wide vnode, kv head); block c serves row pieces c, c + wide_chunks, ..
   int block_slots;                 // blocks of the fused kernel the device runs at a time
@@ -1155,7 +1155,7 @@ __device__ __forceinline__ void merge_shares(float* xchg, WaveState<D, 1>& st, i
   }
 }
 
-// A narrow vnode served by `share` consecutive waves of a block (share = 1, 2, 4 or 8, the same
+// A narrow vnode served by `share` consecutive waves of a block (share = 1, 2 or 4, the same
 // for the whole launch; the host picks more than one when there are fewer vnodes than wave
 // slots): wave w of the vnode takes the tiles w, w + share, ..., and the shares are merged
 // through LDS.  `slot` is the wave's index in the block; a wave without a vnode (exists ==
@@ -1501,8 +1501,8 @@ int launch_stage1_inst(const Stage1Args& a, int hkv, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? FT_OK : FT_ERR_LAUNCH;
 }
 
-// Waves that share one narrow vnode: the largest power of two (at most 8) that fills at most
-// three quarters of the wave slots (8 per compute unit).  With far fewer vnodes than slots the
+// Waves that share one narrow vnode: the largest power of two (at most a block's four) that
+// fills at most three quarters of the wave slots (8 per compute unit).  With far fewer vnodes than slots the
 // waves would each walk a long run alone, one memory round trip per tile; with the slots nearly
 // full the runs are limited by memory bandwidth already and sharing only adds barriers.
 inline int wave_slots() {
