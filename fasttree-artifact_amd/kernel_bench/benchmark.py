@@ -67,20 +67,26 @@ def do_bench(fn, quantiles=QUANTILES, warmup=25, rep=100):
     return torch.quantile(times, torch.tensor(quantiles, dtype=torch.float64)).tolist()
 
 
-def main(args):
-    num_qo_heads, num_kv_heads, head_dim = args.num_qo_heads, args.num_kv_heads, args.head_dim
-    group = num_qo_heads // num_kv_heads
-    dtype = torch.float16
+def planner_options(args):
+    """Query tiles, KV tiles, KV split sizes and the two threshold pairs as lists of int: the
+    options given, else the reference's defaults (kernel_bench/benchmark.py:246-254), else with
+    --mi355x the ones for MI355X."""
+    group = args.num_qo_heads // args.num_kv_heads
     defaults = dict(q_tile_size_per_phase="64,16", kv_split_sizes="1024,128", para_threshs1="132,528", para_threshs2="132,132")
     if args.mi355x:
         defaults = dict(q_tile_size_per_phase=f"{max(1, 64 // group)},{max(1, 16 // group)}", kv_split_sizes="1024,256",
                         para_threshs1="256,1024", para_threshs2="256,256")
     ints = lambda text: list(map(int, text.split(",")))
-    Q_TILE_SIZE_PER_PHASE = ints(args.q_tile_size_per_phase or defaults["q_tile_size_per_phase"])
-    KV_TILE_SIZE_PER_PHASE = ints(args.kv_tile_size_per_phase)
-    KV_SPLIT_SIZES = ints(args.kv_split_sizes or defaults["kv_split_sizes"])
-    para_threshs1 = ints(args.para_threshs1 or defaults["para_threshs1"])
-    para_threshs2 = ints(args.para_threshs2 or defaults["para_threshs2"])
+    return (ints(args.q_tile_size_per_phase or defaults["q_tile_size_per_phase"]), ints(args.kv_tile_size_per_phase),
+            ints(args.kv_split_sizes or defaults["kv_split_sizes"]), ints(args.para_threshs1 or defaults["para_threshs1"]),
+            ints(args.para_threshs2 or defaults["para_threshs2"]))
+
+
+def main(args):
+    num_qo_heads, num_kv_heads, head_dim = args.num_qo_heads, args.num_kv_heads, args.head_dim
+    group = num_qo_heads // num_kv_heads
+    dtype = torch.float16
+    Q_TILE_SIZE_PER_PHASE, KV_TILE_SIZE_PER_PHASE, KV_SPLIT_SIZES, para_threshs1, para_threshs2 = planner_options(args)
 
     params = FastTreeParams()
     params.set_values(args.alpha, args.beta, args.gamma)

@@ -41,6 +41,13 @@ def test_benchmark_options_and_defaults_follow_the_reference():
     assert args.choice == "all" and args.signature is None and args.fasttree_heuristic_path is None and args.profile is False
     assert args.q_tile_size_per_phase is None and args.para_threshs1 is None and args.para_threshs2 is None
     assert args.kv_split_sizes is None
+    assert benchmark.planner_options(args) == ([64, 16], [32, 32], [1024, 128], [132, 528], [132, 132])
+    gqa = ["--load_file_path", "x.txt", "--num_qo_heads", "32", "--num_kv_heads", "8"]
+    assert benchmark.planner_options(benchmark.build_parser().parse_args(gqa + ["--mi355x"])) == (
+        [16, 4], [32, 32], [1024, 256], [256, 1024], [256, 256])
+    # an explicit option wins over --mi355x
+    explicit = benchmark.build_parser().parse_args(gqa + ["--mi355x", "--kv_split_sizes", "512,64", "--para_threshs2", "1,2"])
+    assert benchmark.planner_options(explicit) == ([16, 4], [32, 32], [512, 64], [256, 1024], [1, 2])
     with pytest.raises(SystemExit):
         benchmark.build_parser().parse_args(["--load_file_path", "x.txt", "--choice", "DeFT"])
     with pytest.raises(SystemExit):
