@@ -521,6 +521,98 @@ def vnodes_in_launch_order(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, ph
     return result
 
 
+#: Blocks (128-row blocks x kv heads) the vnodes of one KV run must make for the run's KV split to
+#: be undone: one per compute unit of an MI355X; see :func:`join_kv_chunks`.
+FULL_MACHINE_BLOCKS = 256
+
+
+def join_kv_chunks(kv_offs, kv_lens, q_offs, q_lens, q_entries, req_entries, req_offs, req_lens,
+                   phase_node_nums, phase_node_offsets, group, num_kv_heads, min_blocks=None):
+    """Undoes the KV split of runs whose query rows alone fill the machine.
+
+    The planner cuts every run into chunks of the phase's KV split size whatever the number of
+    requests under it (kernel_bench/fasttree.py:199-231): chunk s of a node is served by its own
+    vnodes over its own copy of the node's scratch rows, and the second stage merges the copies
+    per request.  The split buys parallelism; a run attended by so many query rows that its
+    128-row blocks x kv heads already number ``min_blocks`` (default
+    :data:`FULL_MACHINE_BLOCKS`) has it without the split, and each further chunk then only adds
+    a partial row per request and head to write, read and merge.  For such runs the chunks are
+    joined again: where a vnode's KV slice ends the next chunk's begins (the flat KV index list
+    holds a node's tokens back to back), and when the vnodes over that next slice serve the same
+    requests in the same tiles, the first chunk's vnodes are extended over it and the others are
+    dropped, together with their scratch rows, which leave the per-request lists (the rows
+    stay allocated and unused).  Chains continue over any number of chunks.
+
+    Takes the lists in the planner's order (either phase order is fine) and returns
+    ``(kv_offs, kv_lens, q_offs, q_lens, req_entries, req_offs, req_lens, phase_node_nums,
+    phase_node_offsets)`` with ``req_entries`` padded by 32 x -1 as the planner's
+    (fasttree.py:261-262); the inputs are not modified.
+    """
+    min_blocks = FULL_MACHINE_BLOCKS if min_blocks is None else int(min_blocks)
+    kv_o, kv_l, q_o, q_l = (np.array(x, dtype=np.int64, copy=True) for x in (kv_offs, kv_lens, q_offs, q_lens))
+    q_ent = np.asarray(q_entries, dtype=np.int64)
+    count0 = int(phase_node_nums[0])
+    n = len(kv_o)
+    runs = {}
+    for v in range(n):
+        runs.setdefault((int(kv_o[v]), int(kv_l[v])), []).append(v)
+    starts = {}
+    for key in runs:
+        starts.setdefault(key[0], []).append(key)
+    dropped = np.zeros(n, dtype=bool)
+    absorbed = set()
+    heads = max(1, int(num_kv_heads))
+    for key in sorted(runs):
+        if key in absorbed:
+            continue
+        tiles = runs[key]
+        rows = int(q_l[tiles].sum()) * int(group)
+        if -(-rows // WIDE_BLOCK_ROWS) * heads < min_blocks:
+            continue
+        end = key[0] + key[1]
+        while True:
+            follower = None
+            for cand in starts.get(end, ()):
+                other = runs[cand]
+                if cand in absorbed or cand == key or len(other) != len(tiles):
+                    continue
+                if all(q_l[a] == q_l[b] and (a < count0) == (b < count0)
+                       and np.array_equal(q_ent[q_o[a]: q_o[a] + q_l[a]], q_ent[q_o[b]: q_o[b] + q_l[b]])
+                       for a, b in zip(tiles, other)):
+                    follower = cand
+                    break
+            if follower is None:
+                break
+            absorbed.add(follower)
+            kv_l[tiles] += follower[1]
+            dropped[runs[follower]] = True
+            end = follower[0] + follower[1]
+    entries = np.asarray(req_entries, dtype=np.int64)
+    lens = np.asarray(req_lens, dtype=np.int64)
+    offs = np.asarray(req_offs, dtype=np.int64)
+    total = int(lens.sum())
+    if not dropped.any():
+        return (kv_o.astype(np.int32), kv_l.astype(np.int32), q_o.astype(np.int32), q_l.astype(np.int32),
+                entries.astype(np.int32), offs.astype(np.int32), lens.astype(np.int32),
+                list(phase_node_nums), list(phase_node_offsets))
+    if not np.array_equal(offs, np.concatenate([[0], np.cumsum(lens)[:-1]])):
+        raise ValueError("the per-request lists must lie back to back in request order")
+    row_dropped = np.zeros(len(q_ent), dtype=bool)
+    for v in np.nonzero(dropped)[0]:
+        row_dropped[q_o[v]: q_o[v] + q_l[v]] = True
+    listed = entries[:total]
+    keep = ~row_dropped[listed]
+    owner = np.repeat(np.arange(len(lens)), lens)
+    new_lens = np.bincount(owner[keep], minlength=len(lens))
+    new_offs = np.concatenate([[0], np.cumsum(new_lens)[:-1]])
+    new_entries = np.concatenate([listed[keep], np.full(32, -1, dtype=np.int64)])
+    kept = ~dropped
+    n0 = int(kept[:count0].sum())
+    return (kv_o[kept].astype(np.int32), kv_l[kept].astype(np.int32), q_o[kept].astype(np.int32), q_l[kept].astype(np.int32),
+            new_entries.astype(np.int32), new_offs.astype(np.int32), new_lens.astype(np.int32),
+            [n0, int(kept.sum()) - n0], [0, n0])
+
+
 class PlanBuffers:
     """Device buffers for :func:`fasttree_preparation`, allocated once at stated maxima and
     filled in place by every call that is given them: a serving loop re-plans whenever its batch
@@ -588,8 +680,8 @@ def fasttree_preparation(
     phase_node_offsets), node_assignments)``.  The keyword-only arguments do not exist
     in the reference: ``device`` defaults to the reference's hard-wired "cuda";
     ``kv_slot_map`` is described in :func:`fasttree_plan`; ``launch_order`` arranges the vnodes
-    for the kernels (:func:`vnodes_in_launch_order`) instead of leaving them in the reference's
-    order; with ``buffers`` (a :class:`PlanBuffers`) nothing is allocated on the device: the
+    for the kernels (:func:`join_kv_chunks`, then :func:`vnodes_in_launch_order`) instead of
+    leaving them in the reference's order; with ``buffers`` (a :class:`PlanBuffers`) nothing is allocated on the device: the
     arrays are written into its buffers and the returned tensors are their leading parts.
     """
     import torch
@@ -612,9 +704,12 @@ def fasttree_preparation(
     rows = plan.num_rows
     vnodes = (plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens,
               plan.phase_node_nums, plan.phase_node_offsets)
+    per_request = (plan.req_to_vnode_entries, plan.req_to_vnode_offs, plan.req_to_vnode_lens)
     if launch_order:
-        vnodes = vnodes_in_launch_order(*vnodes, max(1, num_qo_heads // num_kv_heads), num_kv_heads,
-                                        q_tile=params.TSQs[0])
+        group = max(1, num_qo_heads // num_kv_heads)
+        joined = join_kv_chunks(*vnodes[:4], plan.vnode_to_q_entries, *per_request, *vnodes[4:], group, num_kv_heads)
+        vnodes, per_request = (*joined[:4], *joined[7:]), joined[4:7]
+        vnodes = vnodes_in_launch_order(*vnodes, group, num_kv_heads, q_tile=params.TSQs[0])
     if buffers is not None:
         if rows > buffers.mid_o.shape[0] or buffers.mid_o.shape[1:] != (num_qo_heads, head_dim):
             raise ValueError(f"the scratch of the buffers ({tuple(buffers.mid_o.shape)}) does not hold "
@@ -630,9 +725,9 @@ def fasttree_preparation(
         put(plan.vnode_to_q_entries),
         put(vnodes[2]),
         put(vnodes[3]),
-        put(plan.req_to_vnode_entries),
-        put(plan.req_to_vnode_offs),
-        put(plan.req_to_vnode_lens),
+        put(per_request[0]),
+        put(per_request[1]),
+        put(per_request[2]),
         mid_o,
         mid_lse,
         list(vnodes[4]),

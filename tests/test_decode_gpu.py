@@ -399,6 +399,31 @@ def test_wide_vnodes_in_row_chunks_and_uneven_tails(device):
 
 
 @pytest.mark.gpu
+def test_kv_chunks_joined_where_the_rows_fill_the_machine(device, monkeypatch):
+    """1 x 2048 shared tokens under 1024 requests, 32/8 heads: the launch order undoes the root's
+    KV split (4096 query rows fill the machine by themselves), two partial rows per request
+    instead of three; same result as with the planner's own lists, both at the parity bar.  Then
+    forced on a small three-level tree (every chain joined, dropped rows in the middle of the
+    scratch), fp16 and bf16."""
+    from fasttree_hip import planner
+    _announce("kv chunks joined")
+    sample = list(range(0, 1024, 41))
+    aux = _plan_and_check(device, [1, 1024], [2048, 32], 32, 8, 128, [16, 4], [1024, 256], "kv chunks joined",
+                          sample=sample, thr=((256, 1024), (256, 256)))
+    assert aux[8].tolist() == [2] * 1024 and aux[9].shape[0] == 3 * 1024 and max(aux[2].tolist()) == 2048
+    ref = _plan_and_check(device, [1, 1024], [2048, 32], 32, 8, 128, [16, 4], [1024, 256], "kv chunks as planned",
+                          sample=sample, thr=((256, 1024), (256, 256)), launch_order=False)
+    assert ref[8].tolist() == [3] * 1024
+    monkeypatch.setattr(planner, "FULL_MACHINE_BLOCKS", 1)
+    for dtype in (torch.float16, torch.bfloat16):
+        aux = _plan_and_check(device, [1, 4, 36], [700, 300, 45], 16, 4, 128, [16, 4], [256, 64], f"kv chunks forced {dtype}",
+                              dtype=dtype, thr=((10**6, 10**6), (1, 1)))
+        ref = _plan_and_check(device, [1, 4, 36], [700, 300, 45], 16, 4, 128, [16, 4], [256, 64], f"kv chunks as planned {dtype}",
+                              dtype=dtype, thr=((10**6, 10**6), (1, 1)), launch_order=False)
+        assert max(ref[2].tolist()) <= 64 and max(aux[2].tolist()) == 1000 and max(aux[8].tolist()) <= 3 < min(ref[8].tolist())
+
+
+@pytest.mark.gpu
 def test_more_wide_vnodes_than_the_ranking_holds(device):
     """More than 256 wide vnodes: blocks take them in plan order instead of ranking them (the
     planner's own list; in launch order these light vnodes all run with the narrow phase)."""

@@ -206,6 +206,94 @@ def test_launch_order_joins_query_tiles_without_changing_what_is_computed(name):
         assert nums_few == list(plan.phase_node_nums)
 
 
+def _joined_plan(plan, group, hkv, min_blocks):
+    """`plan` with its vnode and per-request lists replaced by what join_kv_chunks returns."""
+    import copy
+    from fasttree_hip.planner import join_kv_chunks
+    out = join_kv_chunks(plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens,
+                         plan.vnode_to_q_entries, plan.req_to_vnode_entries, plan.req_to_vnode_offs, plan.req_to_vnode_lens,
+                         plan.phase_node_nums, plan.phase_node_offsets, group, hkv, min_blocks=min_blocks)
+    new = copy.copy(plan)
+    (new.vnode_to_kv_offs, new.vnode_to_kv_lens, new.vnode_to_q_offs, new.vnode_to_q_lens,
+     new.req_to_vnode_entries, new.req_to_vnode_offs, new.req_to_vnode_lens) = (x.tolist() for x in out[:7])
+    new.phase_node_nums, new.phase_node_offsets = out[7], out[8]
+    return new
+
+
+def _attended(plan, batch):
+    """For each request: the KV index entries the scratch rows *listed for it* attend."""
+    row_vnode = {}
+    for v, (qo, ql) in enumerate(zip(plan.vnode_to_q_offs, plan.vnode_to_q_lens)):
+        for i in range(ql):
+            assert qo + i not in row_vnode, "a scratch row belongs to at most one vnode"
+            row_vnode[qo + i] = v
+    seen = []
+    for r in range(batch):
+        rows = plan.req_to_vnode_entries[plan.req_to_vnode_offs[r]: plan.req_to_vnode_offs[r] + plan.req_to_vnode_lens[r]]
+        assert rows == sorted(set(rows)) and all(plan.vnode_to_q_entries[x] == r for x in rows)
+        got = []
+        for x in rows:
+            v = row_vnode[x]
+            got.extend(range(plan.vnode_to_kv_offs[v], plan.vnode_to_kv_offs[v] + plan.vnode_to_kv_lens[v]))
+        seen.append(sorted(got))
+    assert sorted(row_vnode) == sorted(x for r in range(batch) for x in
+                                       plan.req_to_vnode_entries[plan.req_to_vnode_offs[r]: plan.req_to_vnode_offs[r] + plan.req_to_vnode_lens[r]]), \
+        "every row of a kept vnode is listed for its request, and no dropped row is"
+    return seen
+
+
+@pytest.mark.parametrize("name", ["kat1", "c3", "c5_seed0", "c5_seed1", "shape07_h32_8", "rand03", "rand17", "rand41"])
+def test_joining_kv_chunks_keeps_what_every_request_attends(name):
+    """Forced (one block is enough): every chain of chunks is joined; each request still attends
+    the same entries of the flat KV list, each once, through the rows listed for it; the joined
+    vnodes keep phase and tile widths; the trailing 32 x -1 are there."""
+    case = next(c for c in PLANNER_CASES if c["name"] == name)
+    tree, ptrs, batch, plan, params, _ = run_planner(case)
+    group = case["Hq"] // case["Hkv"]
+    before = _attended(plan, batch)
+    new = _joined_plan(plan, group, case["Hkv"], min_blocks=1)
+    assert _attended(new, batch) == before
+    assert new.req_to_vnode_entries[-32:] == [-1] * 32 and len(new.req_to_vnode_entries) == sum(new.req_to_vnode_lens) + 32
+    wide = new.phase_node_nums[0]
+    assert new.phase_node_offsets == [0, wide] and sum(new.phase_node_nums) == len(new.vnode_to_kv_offs)
+    assert all(n > plan.q_tile_sizes[1] for n in new.vnode_to_q_lens[:wide])
+    assert all(n <= plan.q_tile_sizes[1] for n in new.vnode_to_q_lens[wide:])
+    # nothing left to join: no run (the vnodes over one KV slice) is followed by a run over the same requests in the same tiles
+    runs = {}
+    for ko, kl, qo, ql in zip(new.vnode_to_kv_offs, new.vnode_to_kv_lens, new.vnode_to_q_offs, new.vnode_to_q_lens):
+        runs.setdefault((ko, kl), []).append(tuple(new.vnode_to_q_entries[qo: qo + ql]))
+    for (ko, kl), tiles in runs.items():
+        for (ko2, kl2), tiles2 in runs.items():
+            assert not (ko2 == ko + kl and tiles2 == tiles)
+    if name == "c3":
+        # the root's four chunks become one per query tile: 100 + 30 -> 25 + 30 first-phase vnodes, 3 rows fewer per request
+        assert plan.phase_node_nums == [130, 400] and new.phase_node_nums == [55, 400]
+        assert set(new.req_to_vnode_lens) == {3} and set(plan.req_to_vnode_lens) == {6}
+    # the inputs are untouched, and with the default threshold small trees stay as they are
+    same = _joined_plan(plan, group, case["Hkv"], min_blocks=None)
+    if name != "c5_seed0" and name != "c5_seed1":
+        assert same.vnode_to_kv_lens == list(plan.vnode_to_kv_lens) and same.req_to_vnode_entries == list(plan.req_to_vnode_entries)
+
+
+def test_joining_kv_chunks_only_where_the_rows_fill_the_machine():
+    """1 x 2048 shared tokens under 1024 requests, 32/8 heads: 4096 query rows = 32 blocks x 8 kv
+    heads = 256 blocks without the split, so the root's two chunks are joined; under 256 requests
+    (64 blocks) they are not."""
+    from fasttree_hip.planner import FastTreeParams, fasttree_plan
+    for leaves, joins in ((1024, True), (256, False)):
+        tree, ptrs, batch = build_tree({"kind": "regular", "sizes": [1, leaves], "lens": [2048, 32]})
+        p = FastTreeParams(); p.set_values(0.66, 0.33, 0.1); p.set_q_tile_sizes([16, 4]); p.set_kv_tile_sizes([32, 32]); p.set_kv_group_num(4)
+        plan = fasttree_plan(tree, ptrs, batch, 8, [1024, 256], [256, 1024], [256, 256], p)
+        assert plan.phase_node_nums == [2 * leaves // 16, leaves] and set(plan.req_to_vnode_lens) == {3}
+        new = _joined_plan(plan, 4, 8, None)
+        if joins:
+            assert new.phase_node_nums == [leaves // 16, leaves] and set(new.req_to_vnode_lens) == {2}
+            assert set(new.vnode_to_kv_lens[:leaves // 16]) == {2048}
+        else:
+            assert new.phase_node_nums == plan.phase_node_nums and new.vnode_to_kv_lens == list(plan.vnode_to_kv_lens)
+        assert _attended(new, batch) == _attended(plan, batch)
+
+
 def test_preparation_into_preallocated_buffers():
     """fasttree_preparation(buffers=...) writes into the same device buffers on every call and
     returns their leading parts; the contents equal those of the allocating call."""
