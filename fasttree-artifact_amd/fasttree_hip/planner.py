@@ -550,18 +550,33 @@ def join_kv_chunks(kv_offs, kv_lens, q_offs, q_lens, q_entries, req_entries, req
     """
     min_blocks = FULL_MACHINE_BLOCKS if min_blocks is None else int(min_blocks)
     kv_o, kv_l, q_o, q_l = (np.array(x, dtype=np.int64, copy=True) for x in (kv_offs, kv_lens, q_offs, q_lens))
+    heads = max(1, int(num_kv_heads))
+
+    def unchanged():
+        return (kv_o.astype(np.int32), kv_l.astype(np.int32), q_o.astype(np.int32), q_l.astype(np.int32),
+                np.asarray(req_entries, dtype=np.int32), np.asarray(req_offs, dtype=np.int32),
+                np.asarray(req_lens, dtype=np.int32), list(phase_node_nums), list(phase_node_offsets))
+
+    # (most launches have no such run: requests per run, summed over its vnodes)
+    _, run_of = np.unique((kv_o << 32) | kv_l, return_inverse=True)
+    run_rows = np.bincount(run_of, weights=q_l).astype(np.int64) * int(group)
+    big = (-(-run_rows // WIDE_BLOCK_ROWS) * heads >= min_blocks)[run_of]
+    if not big.any():
+        return unchanged()
     q_ent = np.asarray(q_entries, dtype=np.int64)
     count0 = int(phase_node_nums[0])
     n = len(kv_o)
+    # candidates: the vnodes of the big runs, and every vnode that begins where one of those ends
+    ends = set((kv_o[big] + kv_l[big]).tolist())
     runs = {}
     for v in range(n):
-        runs.setdefault((int(kv_o[v]), int(kv_l[v])), []).append(v)
+        if big[v] or int(kv_o[v]) in ends:
+            runs.setdefault((int(kv_o[v]), int(kv_l[v])), []).append(v)
     starts = {}
     for key in runs:
         starts.setdefault(key[0], []).append(key)
     dropped = np.zeros(n, dtype=bool)
     absorbed = set()
-    heads = max(1, int(num_kv_heads))
     for key in sorted(runs):
         if key in absorbed:
             continue
@@ -587,14 +602,12 @@ def join_kv_chunks(kv_offs, kv_lens, q_offs, q_lens, q_entries, req_entries, req
             kv_l[tiles] += follower[1]
             dropped[runs[follower]] = True
             end = follower[0] + follower[1]
+    if not dropped.any():
+        return unchanged()
     entries = np.asarray(req_entries, dtype=np.int64)
     lens = np.asarray(req_lens, dtype=np.int64)
     offs = np.asarray(req_offs, dtype=np.int64)
     total = int(lens.sum())
-    if not dropped.any():
-        return (kv_o.astype(np.int32), kv_l.astype(np.int32), q_o.astype(np.int32), q_l.astype(np.int32),
-                entries.astype(np.int32), offs.astype(np.int32), lens.astype(np.int32),
-                list(phase_node_nums), list(phase_node_offsets))
     if not np.array_equal(offs, np.concatenate([[0], np.cumsum(lens)[:-1]])):
         raise ValueError("the per-request lists must lie back to back in request order")
     row_dropped = np.zeros(len(q_ent), dtype=bool)
