@@ -525,71 +525,87 @@ def vnodes_in_launch_order(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, ph
 #: be undone: one per compute unit of an MI355X; see :func:`join_kv_chunks`.
 FULL_MACHINE_BLOCKS = 256
 
+#: First-phase blocks a launch may have for all of them to be resident at once with a few block
+#: slots to spare (of :data:`WIDE_BLOCK_SLOTS`); see :func:`join_kv_chunks`.
+RESIDENT_WIDE_BLOCKS = 472
+
 
 def join_kv_chunks(kv_offs, kv_lens, q_offs, q_lens, q_entries, req_entries, req_offs, req_lens,
-                   phase_node_nums, phase_node_offsets, group, num_kv_heads, min_blocks=None):
-    """Undoes the KV split of runs whose query rows alone fill the machine.
+                   phase_node_nums, phase_node_offsets, group, num_kv_heads, min_blocks=None, resident_blocks=None):
+    """Cuts long KV runs into fewer chunks than the planner did where the chunks buy nothing.
 
     The planner cuts every run into chunks of the phase's KV split size whatever the number of
     requests under it (kernel_bench/fasttree.py:199-231): chunk s of a node is served by its own
     vnodes over its own copy of the node's scratch rows, and the second stage merges the copies
-    per request.  The split buys parallelism; a run attended by so many query rows that its
-    128-row blocks x kv heads already number ``min_blocks`` (default
-    :data:`FULL_MACHINE_BLOCKS`) has it without the split, and each further chunk then only adds
-    a partial row per request and head to write, read and merge.  For such runs the chunks are
-    joined again: where a vnode's KV slice ends the next chunk's begins (the flat KV index list
-    holds a node's tokens back to back), and when the vnodes over that next slice serve the same
-    requests in the same tiles, the first chunk's vnodes are extended over it and the others are
-    dropped, together with their scratch rows, which leave the per-request lists (the rows
-    stay allocated and unused).  Chains continue over any number of chunks.
+    per request.  The split buys parallelism, and each chunk costs a partial row per request and
+    head to write, read and merge.  Two cases where fewer chunks are better:
 
-    Takes the lists in the planner's order (either phase order is fine) and returns
+    * a run attended by so many query rows that the 128-row blocks x kv heads of ONE chunk
+      already number ``min_blocks`` (default :data:`FULL_MACHINE_BLOCKS`) has its parallelism
+      without the split: it becomes one chunk;
+    * a launch whose first phase has a few more blocks than the machine holds at once
+      (``resident_blocks``, default :data:`RESIDENT_WIDE_BLOCKS`) runs its last blocks behind the
+      others and keeps the second phase's short vnodes waiting for a block slot; when giving the
+      chunked runs fewer chunks brings the first phase under that number, the largest runs get
+      the most chunks that fit (C3: three chunks of its 4000-token root instead of four,
+      472 blocks instead of 576).
+
+    Where a vnode's KV slice ends the next chunk's begins (the flat KV index list holds a node's
+    tokens back to back); vnodes over that next slice that serve the same requests in the same
+    tiles are the next chunk.  A chain of S chunks that is to have S' < S is cut anew into S'
+    equal slices (multiples of 64 tokens) served by the vnodes of its first S' chunks; the vnodes
+    of the others are dropped together with their scratch rows, which leave the per-request
+    lists (the rows stay allocated and unused).
+
+    Takes the lists in the planner's order (first phase, then second) and returns
     ``(kv_offs, kv_lens, q_offs, q_lens, req_entries, req_offs, req_lens, phase_node_nums,
     phase_node_offsets)`` with ``req_entries`` padded by 32 x -1 as the planner's
     (fasttree.py:261-262); the inputs are not modified.
     """
     min_blocks = FULL_MACHINE_BLOCKS if min_blocks is None else int(min_blocks)
+    resident = RESIDENT_WIDE_BLOCKS if resident_blocks is None else int(resident_blocks)
     kv_o, kv_l, q_o, q_l = (np.array(x, dtype=np.int64, copy=True) for x in (kv_offs, kv_lens, q_offs, q_lens))
     heads = max(1, int(num_kv_heads))
+    count0 = int(phase_node_nums[0])
+    n = len(kv_o)
 
     def unchanged():
         return (kv_o.astype(np.int32), kv_l.astype(np.int32), q_o.astype(np.int32), q_l.astype(np.int32),
                 np.asarray(req_entries, dtype=np.int32), np.asarray(req_offs, dtype=np.int32),
                 np.asarray(req_lens, dtype=np.int32), list(phase_node_nums), list(phase_node_offsets))
 
-    # (most launches have no such run: requests per run, summed over its vnodes)
-    _, run_of = np.unique((kv_o << 32) | kv_l, return_inverse=True)
+    if n == 0:
+        return unchanged()
+    # blocks per run (the vnodes over one KV slice): requests summed over its vnodes
+    _, first_of, run_of = np.unique((kv_o << 32) | kv_l, return_index=True, return_inverse=True)
     run_rows = np.bincount(run_of, weights=q_l).astype(np.int64) * int(group)
-    big = (-(-run_rows // WIDE_BLOCK_ROWS) * heads >= min_blocks)[run_of]
-    if not big.any():
+    run_blocks = -(-run_rows // WIDE_BLOCK_ROWS) * heads
+    wide_total = int(run_blocks[first_of < count0].sum())  # (a run's vnodes share a phase but for a narrow last tile)
+    full = run_blocks >= min_blocks
+    if not full.any() and wide_total <= resident:
+        return unchanged()
+    # candidates: runs that another run follows or that follow another run
+    run_start, run_end = kv_o[first_of], kv_o[first_of] + kv_l[first_of]
+    chained = np.isin(run_end, run_start) | np.isin(run_start, run_end)
+    if not chained.any():
         return unchanged()
     q_ent = np.asarray(q_entries, dtype=np.int64)
-    count0 = int(phase_node_nums[0])
-    n = len(kv_o)
-    # candidates: the vnodes of the big runs, and every vnode that begins where one of those ends
-    ends = set((kv_o[big] + kv_l[big]).tolist())
     runs = {}
-    for v in range(n):
-        if big[v] or int(kv_o[v]) in ends:
-            runs.setdefault((int(kv_o[v]), int(kv_l[v])), []).append(v)
+    for v in np.nonzero(chained[run_of])[0].tolist():
+        runs.setdefault((int(kv_o[v]), int(kv_l[v])), []).append(v)
     starts = {}
     for key in runs:
         starts.setdefault(key[0], []).append(key)
-    dropped = np.zeros(n, dtype=bool)
-    absorbed = set()
+    chains, taken = [], set()
     for key in sorted(runs):
-        if key in absorbed:
+        if key in taken:
             continue
-        tiles = runs[key]
-        rows = int(q_l[tiles].sum()) * int(group)
-        if -(-rows // WIDE_BLOCK_ROWS) * heads < min_blocks:
-            continue
-        end = key[0] + key[1]
+        chain, tiles, end = [key], runs[key], key[0] + key[1]
         while True:
             follower = None
             for cand in starts.get(end, ()):
                 other = runs[cand]
-                if cand in absorbed or cand == key or len(other) != len(tiles):
+                if cand in taken or cand == key or len(other) != len(tiles):
                     continue
                 if all(q_l[a] == q_l[b] and (a < count0) == (b < count0)
                        and np.array_equal(q_ent[q_o[a]: q_o[a] + q_l[a]], q_ent[q_o[b]: q_o[b] + q_l[b]])
@@ -598,10 +614,42 @@ def join_kv_chunks(kv_offs, kv_lens, q_offs, q_lens, q_entries, req_entries, req
                     break
             if follower is None:
                 break
-            absorbed.add(follower)
-            kv_l[tiles] += follower[1]
-            dropped[runs[follower]] = True
+            taken.add(follower)
+            chain.append(follower)
             end = follower[0] + follower[1]
+        if len(chain) > 1:
+            rows = int(q_l[tiles].sum()) * int(group)
+            chains.append((-(-rows // WIDE_BLOCK_ROWS) * heads, chain))
+    # how many chunks each chain keeps
+    plan = []
+    for per, chain in chains:
+        if per >= min_blocks:
+            plan.append((per, chain, 1))
+            if runs[chain[0]][0] < count0:
+                wide_total -= per * (len(chain) - 1)
+    if wide_total > resident:
+        rest = [(per, chain) for per, chain in chains if per < min_blocks and runs[chain[0]][0] < count0]
+        spare = sum(per * (len(chain) - 1) for per, chain in rest)
+        if wide_total - spare <= resident:  # fewer chunks can bring the phase under the number
+            for per, chain in sorted(rest, key=lambda x: -x[0] * len(x[1])):
+                others = wide_total - per * len(chain)
+                keep = min(len(chain), max(1, (resident - others) // per))
+                if keep < len(chain):
+                    plan.append((per, chain, keep))
+                    wide_total = others + per * keep
+                if wide_total <= resident:
+                    break
+    dropped = np.zeros(n, dtype=bool)
+    for per, chain, keep in plan:
+        start = chain[0][0]
+        total = sum(key[1] for key in chain)
+        size = -(-(-(-total // keep)) // 64) * 64  # ceil(total / keep), up to a multiple of 64
+        for i, key in enumerate(chain):
+            if i < keep and i * size < total:
+                kv_o[runs[key]] = start + i * size
+                kv_l[runs[key]] = min(size, total - i * size)
+            else:
+                dropped[runs[key]] = True
     if not dropped.any():
         return unchanged()
     entries = np.asarray(req_entries, dtype=np.int64)

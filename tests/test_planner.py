@@ -269,10 +269,36 @@ def test_joining_kv_chunks_keeps_what_every_request_attends(name):
         # the root's four chunks become one per query tile: 100 + 30 -> 25 + 30 first-phase vnodes, 3 rows fewer per request
         assert plan.phase_node_nums == [130, 400] and new.phase_node_nums == [55, 400]
         assert set(new.req_to_vnode_lens) == {3} and set(plan.req_to_vnode_lens) == {6}
-    # the inputs are untouched, and with the default threshold small trees stay as they are
+    # the inputs are untouched; with the default thresholds small trees stay as they are, and C3's root gets three
+    # chunks of 1344, 1344 and 1312 tokens instead of four (3 x 104 + 160 = 472 first-phase blocks instead of 576)
     same = _joined_plan(plan, group, case["Hkv"], min_blocks=None)
-    if name != "c5_seed0" and name != "c5_seed1":
+    assert _attended(same, batch) == before
+    if name == "c3":
+        assert same.phase_node_nums == [3 * 25 + 30, 400] and set(same.req_to_vnode_lens) == {5}
+        assert sorted(set(same.vnode_to_kv_lens[:75])) == [1312, 1344] and same.vnode_to_kv_offs[50] == 2688
+    elif name not in ("c5_seed0", "c5_seed1"):
         assert same.vnode_to_kv_lens == list(plan.vnode_to_kv_lens) and same.req_to_vnode_entries == list(plan.req_to_vnode_entries)
+
+
+def test_kv_chunks_are_cut_anew_to_fit_the_first_phase_into_the_machine():
+    """C3 (root: 104 blocks per chunk, four chunks; the level below: 160 blocks): the root keeps
+    the most chunks that bring the first phase under the number of resident blocks, or all four
+    when no number of chunks does."""
+    from fasttree_hip.planner import join_kv_chunks
+    case = next(c for c in PLANNER_CASES if c["name"] == "c3")
+    tree, ptrs, batch, plan, params, _ = run_planner(case)
+    before = _attended(plan, batch)
+    for resident, chunks in ((10**9, 4), (576, 4), (575, 3), (472, 3), (471, 2), (368, 2), (367, 1), (264, 1), (263, 4)):
+        out = join_kv_chunks(plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens,
+                             plan.vnode_to_q_entries, plan.req_to_vnode_entries, plan.req_to_vnode_offs, plan.req_to_vnode_lens,
+                             plan.phase_node_nums, plan.phase_node_offsets, 4, 8, resident_blocks=resident)
+        assert out[7] == [25 * chunks + 30, 400], (resident, out[7])
+        assert set(out[6].tolist()) == {chunks + 2}
+        root = sorted(set(zip(out[0][:25 * chunks].tolist(), out[1][:25 * chunks].tolist())))
+        assert len(root) == chunks and root[0][0] == 0 and sum(n for _, n in root) == 4000
+        assert all(a + n == b for (a, n), (b, _) in zip(root, root[1:])) and all(n % 64 == 0 for _, n in root[:-1])
+        new = _joined_plan(plan, 4, 8, None)
+        assert _attended(new, batch) == before
 
 
 def test_joining_kv_chunks_only_where_the_rows_fill_the_machine():
