@@ -58,7 +58,7 @@ WORKLOADS = {
 # HBM bytes per stage-1 launch (read + write) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
 # each scaled by what the same counter reads for a plain copy of known size (2.000 and 1.000); the
 # runs and their commands are summarised in profiles/stage1_fused_stage2_<workload>_<dtype>.txt.
-MEASURED_TRAFFIC = {("c3", "mi355x", "stage1"): 161.0e6, ("c4", "mi355x", "stage1"): 8715.3e6}
+MEASURED_TRAFFIC = {("c3", "mi355x", "stage1"): 140.7e6, ("c4", "mi355x", "stage1"): 8715.3e6}
 
 PRESETS = {
     "reference": dict(q_tiles=None, kv_tiles=(32, 32), kv_splits=(1024, 128), thr1=(132, 528), thr2=(132, 132)),
