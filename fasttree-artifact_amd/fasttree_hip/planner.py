@@ -531,7 +531,8 @@ RESIDENT_WIDE_BLOCKS = 472
 
 
 def join_kv_chunks(kv_offs, kv_lens, q_offs, q_lens, q_entries, req_entries, req_offs, req_lens,
-                   phase_node_nums, phase_node_offsets, group, num_kv_heads, min_blocks=None, resident_blocks=None):
+                   phase_node_nums, phase_node_offsets, group, num_kv_heads, min_blocks=None, resident_blocks=None,
+                   return_order=False):
     """Cuts long KV runs into fewer chunks than the planner did where the chunks buy nothing.
 
     The planner cuts every run into chunks of the phase's KV split size whatever the number of
@@ -560,7 +561,8 @@ def join_kv_chunks(kv_offs, kv_lens, q_offs, q_lens, q_entries, req_entries, req
     Takes the lists in the planner's order (first phase, then second) and returns
     ``(kv_offs, kv_lens, q_offs, q_lens, req_entries, req_offs, req_lens, phase_node_nums,
     phase_node_offsets)`` with ``req_entries`` padded by 32 x -1 as the planner's
-    (fasttree.py:261-262); the inputs are not modified.
+    (fasttree.py:261-262); the inputs are not modified.  With ``return_order`` a tenth
+    element: for every vnode of the input its position in the output, or -1 if it was dropped.
     """
     min_blocks = FULL_MACHINE_BLOCKS if min_blocks is None else int(min_blocks)
     resident = RESIDENT_WIDE_BLOCKS if resident_blocks is None else int(resident_blocks)
@@ -570,9 +572,10 @@ def join_kv_chunks(kv_offs, kv_lens, q_offs, q_lens, q_entries, req_entries, req
     n = len(kv_o)
 
     def unchanged():
-        return (kv_o.astype(np.int32), kv_l.astype(np.int32), q_o.astype(np.int32), q_l.astype(np.int32),
-                np.asarray(req_entries, dtype=np.int32), np.asarray(req_offs, dtype=np.int32),
-                np.asarray(req_lens, dtype=np.int32), list(phase_node_nums), list(phase_node_offsets))
+        out = (kv_o.astype(np.int32), kv_l.astype(np.int32), q_o.astype(np.int32), q_l.astype(np.int32),
+               np.asarray(req_entries, dtype=np.int32), np.asarray(req_offs, dtype=np.int32),
+               np.asarray(req_lens, dtype=np.int32), list(phase_node_nums), list(phase_node_offsets))
+        return (*out, np.arange(n, dtype=np.int64)) if return_order else out
 
     if n == 0:
         return unchanged()
@@ -669,9 +672,14 @@ def join_kv_chunks(kv_offs, kv_lens, q_offs, q_lens, q_entries, req_entries, req
     new_entries = np.concatenate([listed[keep], np.full(32, -1, dtype=np.int64)])
     kept = ~dropped
     n0 = int(kept[:count0].sum())
-    return (kv_o[kept].astype(np.int32), kv_l[kept].astype(np.int32), q_o[kept].astype(np.int32), q_l[kept].astype(np.int32),
-            new_entries.astype(np.int32), new_offs.astype(np.int32), new_lens.astype(np.int32),
-            [n0, int(kept.sum()) - n0], [0, n0])
+    out = (kv_o[kept].astype(np.int32), kv_l[kept].astype(np.int32), q_o[kept].astype(np.int32), q_l[kept].astype(np.int32),
+           new_entries.astype(np.int32), new_offs.astype(np.int32), new_lens.astype(np.int32),
+           [n0, int(kept.sum()) - n0], [0, n0])
+    if return_order:
+        where = np.full(n, -1, dtype=np.int64)
+        where[kept] = np.arange(int(kept.sum()))
+        out = (*out, where)
+    return out
 
 
 class PlanBuffers:

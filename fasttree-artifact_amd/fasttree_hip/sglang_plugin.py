@@ -22,6 +22,7 @@ from collections import defaultdict, deque
 from types import MethodType
 from typing import Dict, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 
@@ -273,15 +274,29 @@ def prepare_for_fasttree_meta(batch, fasttree_metadata: FastTreeMetadata):
     meta.phase_node_offsets = [0, len(above)]
     lists = [[x[i] for i in perm] for x in (kv_offs, kv_lens, q_offs, q_lens)]
     if getattr(meta, "launch_order", False):
-        from .planner import vnodes_in_launch_order
+        from .planner import join_kv_chunks, vnodes_in_launch_order
 
+        # long shared runs in fewer KV chunks where the chunks buy nothing (a system prompt under
+        # a large batch), then the vnodes in launch order
+        tail_ends = [lists[0][v] + lists[1][v] for v in meta.req_last_vnodes]
+        *lists, req_entries, req_offs, req_lens, nums, offs, kept = join_kv_chunks(
+            *lists, q_entries, req_entries, req_offs, req_lens, meta.phase_node_nums, meta.phase_node_offsets,
+            meta.kv_group_num, meta.num_kv_heads, return_order=True)
+        req_entries, req_offs, req_lens = req_entries[: int(np.sum(req_lens))].tolist(), req_offs.tolist(), req_lens.tolist()
+        # a request's last vnode is the single-request vnode that ends where its tokens end; when
+        # that one went with a chunk, the vnode its chain was given to ends there now
+        ends_of = {}
+        for v, (ko, kl, qo, ql) in enumerate(zip(*(x.tolist() for x in lists))):
+            if ql == 1:
+                ends_of[(ko + kl, q_entries[qo])] = v
+        last = [int(kept[v]) if kept[v] >= 0 else ends_of[(end, rid)]
+                for rid, (v, end) in enumerate(zip(meta.req_last_vnodes, tail_ends))]
         *arranged, nums, offs, where = vnodes_in_launch_order(
-            *lists, meta.phase_node_nums, meta.phase_node_offsets, meta.kv_group_num, meta.num_kv_heads,
-            q_tile=q_tiles[0], return_order=True)
+            *lists, nums, offs, meta.kv_group_num, meta.num_kv_heads, q_tile=q_tiles[0], return_order=True)
         lists = [x.tolist() for x in arranged]
         meta.phase_node_nums, meta.phase_node_offsets = nums, offs
-        # (the tail vnodes are single-request vnodes of the second phase: never absorbed)
-        meta.req_last_vnodes = [int(where[v]) for v in meta.req_last_vnodes]
+        # (single-request vnodes of the second phase are never absorbed as query tiles)
+        meta.req_last_vnodes = [int(where[v]) for v in last]
 
     def upload(dst, values):
         src = torch.tensor(values, device="cpu", dtype=torch.int32)

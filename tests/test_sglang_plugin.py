@@ -83,9 +83,11 @@ def make_batch(prompts, outputs, shared_prefixes, device="cpu", max_ctx=64, row_
 def plan_lists(meta, batch):
     nv = sum(meta.phase_node_nums)
     rows = int(meta.req_to_vnode_offs[len(batch.reqs) - 1] + meta.req_to_vnode_lens[len(batch.reqs) - 1])
+    # (rows of chunks the launch order dropped stay in the scratch, unlisted: the rows that are in use may end later)
+    used = max(rows, int((meta.vnode_to_q_offs[:nv] + meta.vnode_to_q_lens[:nv]).max()))
     return dict(kv_offs=meta.vnode_to_kv_offs[:nv].tolist(), kv_lens=meta.vnode_to_kv_lens[:nv].tolist(),
                 q_offs=meta.vnode_to_q_offs[:nv].tolist(), q_lens=meta.vnode_to_q_lens[:nv].tolist(),
-                q_entries=meta.vnode_to_q_entries[:rows].tolist(), req_entries=meta.req_to_vnode_entries[:rows].tolist(),
+                q_entries=meta.vnode_to_q_entries[:used].tolist(), req_entries=meta.req_to_vnode_entries[:rows].tolist(),
                 req_offs=meta.req_to_vnode_offs[: len(batch.reqs)].tolist(),
                 req_lens=meta.req_to_vnode_lens[: len(batch.reqs)].tolist())
 
@@ -187,6 +189,57 @@ def test_every_token_is_covered_once(seed):
         assert all(got["q_entries"][i] == r for i in rows) and rows == sorted(rows)
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2, 3, 4, 5])
+def test_chunk_joins_keep_the_coverage_and_the_last_vnodes(seed, monkeypatch):
+    """The launch order's chunk rule forced on every chain (system prompt, group prefixes,
+    prompts and generated tails all longer than the KV split): every request still attends each
+    of its tokens once through the rows listed for it, its last vnode is a single-request vnode
+    that ends where its tokens end, and the in-place step makes it cover the next token."""
+    from fasttree_hip import planner
+    rng = random.Random(100 + seed)
+    system = [rng.randint(1, 10**6) for _ in range(rng.randint(20, 60))]
+    prefixes, prompts, outputs = [system], [], []
+    for _ in range(rng.randint(1, 3)):
+        mid = system + [rng.randint(1, 10**6) for _ in range(rng.randint(1, 40))]
+        prefixes.append(mid)
+        for _ in range(rng.randint(1, 20)):
+            prompts.append(mid + [rng.randint(1, 10**6) for _ in range(rng.randint(1, 30))])
+            outputs.append([rng.randint(1, 10**6) for _ in range(rng.randint(0, 25))])
+    batch, _ = make_batch(prompts, outputs, prefixes, max_ctx=256)
+    plain = small_meta(kv_split_sizes=(8, 8), launch_order=False)
+    prepare_for_fasttree_meta(batch, plain)
+    monkeypatch.setattr(planner, "FULL_MACHINE_BLOCKS", 1)
+    meta = small_meta(kv_split_sizes=(8, 8))
+    prepare_for_fasttree_meta(batch, meta)
+    assert sum(meta.phase_node_nums) < sum(plain.phase_node_nums), "chunks were joined"
+    table = batch.req_to_token_pool.req_to_token
+    got = plan_lists(meta, batch)
+    flat = table.reshape(-1)
+    row_vnode = {}
+    for v, (qo, ql) in enumerate(zip(got["q_offs"], got["q_lens"])):
+        for i in range(ql):
+            assert qo + i not in row_vnode
+            row_vnode[qo + i] = v
+    listed = set()
+    for r, (p, o) in enumerate(zip(prompts, outputs)):
+        rows = got["req_entries"][got["req_offs"][r]: got["req_offs"][r] + got["req_lens"][r]]
+        assert rows == sorted(set(rows)) and all(got["q_entries"][i] == r for i in rows)
+        listed.update(rows)
+        seen = []
+        for i in rows:
+            v = row_vnode[i]
+            seen += flat[got["kv_offs"][v]: got["kv_offs"][v] + got["kv_lens"][v]].tolist()
+        assert sorted(seen) == sorted(table[r, : len(p) + len(o) + 1].tolist())
+        v = meta.req_last_vnodes[r]
+        assert got["q_lens"][v] == 1 and got["q_entries"][got["q_offs"][v]] == r
+        assert got["kv_offs"][v] + got["kv_lens"][v] == r * table.stride(0) + len(p) + len(o) + 1
+    assert listed == set(row_vnode), "no row of a kept vnode is unlisted, no dropped row is listed"
+    before = meta.vnode_to_kv_lens[: sum(meta.phase_node_nums)].clone()
+    prepare_for_fasttree_step(batch, meta)
+    grown = meta.vnode_to_kv_lens[: sum(meta.phase_node_nums)] - before
+    assert grown.sum().item() == len(prompts) and all(grown[v].item() == 1 for v in meta.req_last_vnodes)
+
+
 def test_annotate_function_keeps_results_and_errors():
     """The breakdown wrapper of load_fasttree_plugin(annotate_breakdown=True): same result, same
     exception, the original reachable, the range closed either way."""
@@ -232,9 +285,13 @@ class FakePool:
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("joined", [False, True])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_hook_matches_dense_attention(device, dtype):
+def test_hook_matches_dense_attention(device, dtype, joined, monkeypatch):
+    """`joined`: 32-token KV splits with the launch order's chunk rule forced on every chain, so
+    that the step after it grows vnodes that were given other vnodes' chunks."""
     import fasttree_oracle as oracle
+    from fasttree_hip import planner
     from helpers import assert_parity
 
     rng = random.Random(7)
@@ -251,8 +308,13 @@ def test_hook_matches_dense_attention(device, dtype):
     rows = list(range(n))
     rng.shuffle(rows)
     batch, n_slots = make_batch(prompts, outputs, prefixes, device=device, max_ctx=256, row_of=rows)
-    meta = small_meta(device=device, TSQs=(256 // 4, 16 // 4))
+    if joined:
+        monkeypatch.setattr(planner, "FULL_MACHINE_BLOCKS", 1)
+        meta = small_meta(device=device, TSQs=(256 // 4, 16 // 4), kv_split_sizes=(32, 16))
+    else:
+        meta = small_meta(device=device, TSQs=(256 // 4, 16 // 4))
     prepare_for_fasttree_meta(batch, meta)
+    print("\n[gpu case] hook", dtype, "joined" if joined else "as planned", "vnodes", list(meta.phase_node_nums), flush=True)
 
     g = torch.Generator().manual_seed(3)
     k_pool = torch.randn((n_slots + 8, hkv, d), generator=g).to(dtype).to(device)
