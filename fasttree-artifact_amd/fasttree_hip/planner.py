@@ -546,10 +546,12 @@ def join_kv_chunks(kv_offs, kv_lens, q_offs, q_lens, q_entries, req_entries, req
       without the split: it becomes one chunk;
     * a launch whose first phase has a few more blocks than the machine holds at once
       (``resident_blocks``, default :data:`RESIDENT_WIDE_BLOCKS`) runs its last blocks behind the
-      others and keeps the second phase's short vnodes waiting for a block slot; when giving the
-      chunked runs fewer chunks brings the first phase under that number, the largest runs get
-      the most chunks that fit (C3: three chunks of its 4000-token root instead of four,
-      472 blocks instead of 576).
+      others and keeps the second phase's short vnodes waiting for a block slot; when longer
+      chunks bring the first phase under that number, the chunked runs are cut at the shortest
+      common chunk length that does (C3: three chunks of its 4000-token root instead of four,
+      472 blocks instead of 576).  Only runs whose blocks still number nine tenths of
+      ``min_blocks`` afterwards are cut anew: a few long blocks on an otherwise idle machine
+      would cost more.
 
     Where a vnode's KV slice ends the next chunk's begins (the flat KV index list holds a node's
     tokens back to back); vnodes over that next slice that serve the same requests in the same
@@ -631,17 +633,27 @@ def join_kv_chunks(kv_offs, kv_lens, q_offs, q_lens, q_entries, req_entries, req
             if runs[chain[0]][0] < count0:
                 wide_total -= per * (len(chain) - 1)
     if wide_total > resident:
-        rest = [(per, chain) for per, chain in chains if per < min_blocks and runs[chain[0]][0] < count0]
-        spare = sum(per * (len(chain) - 1) for per, chain in rest)
-        if wide_total - spare <= resident:  # fewer chunks can bring the phase under the number
-            for per, chain in sorted(rest, key=lambda x: -x[0] * len(x[1])):
-                others = wide_total - per * len(chain)
-                keep = min(len(chain), max(1, (resident - others) // per))
-                if keep < len(chain):
-                    plan.append((per, chain, keep))
-                    wide_total = others + per * keep
-                if wide_total <= resident:
-                    break
+        # One chunk length for all: the shortest for which the phase fits, every run that is cut
+        # anew still covering the machine by itself (its blocks number nine tenths of min_blocks
+        # or more; runs that cannot are left as they are -- a few long blocks on an otherwise
+        # idle machine would be what the launch waits for).
+        covering = max(1, 9 * min_blocks // 10)
+        rest = []
+        for per, chain in chains:
+            fewest = -(-covering // per)
+            if per < min_blocks and runs[chain[0]][0] < count0 and fewest < len(chain):
+                rest.append((per, chain, sum(key[1] for key in chain), fewest))
+        fixed = wide_total - sum(per * len(chain) for per, chain, _, _ in rest)
+
+        def chunks_at(length):
+            return [min(len(chain), max(fewest, -(-tokens // length))) for _, chain, tokens, fewest in rest]
+
+        lengths = sorted({-(-tokens // k) for _, chain, tokens, fewest in rest for k in range(fewest, len(chain) + 1)})
+        for length in lengths:
+            keeps = chunks_at(length)
+            if fixed + sum(per * keep for (per, _, _, _), keep in zip(rest, keeps)) <= resident:
+                plan += [(per, chain, keep) for (per, chain, _, _), keep in zip(rest, keeps) if keep < len(chain)]
+                break
     dropped = np.zeros(n, dtype=bool)
     for per, chain, keep in plan:
         start = chain[0][0]

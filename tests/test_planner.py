@@ -281,24 +281,41 @@ def test_joining_kv_chunks_keeps_what_every_request_attends(name):
 
 
 def test_kv_chunks_are_cut_anew_to_fit_the_first_phase_into_the_machine():
-    """C3 (root: 104 blocks per chunk, four chunks; the level below: 160 blocks): the root keeps
-    the most chunks that bring the first phase under the number of resident blocks, or all four
-    when no number of chunks does."""
+    """C3 (root: 104 blocks per chunk, four chunks; the level below: 160 blocks): the root is cut
+    at the shortest chunk length that brings the first phase under the number of resident
+    blocks, as long as its own blocks still number nine tenths of `min_blocks`; else it keeps its four chunks."""
     from fasttree_hip.planner import join_kv_chunks
     case = next(c for c in PLANNER_CASES if c["name"] == "c3")
     tree, ptrs, batch, plan, params, _ = run_planner(case)
     before = _attended(plan, batch)
-    for resident, chunks in ((10**9, 4), (576, 4), (575, 3), (472, 3), (471, 2), (368, 2), (367, 1), (264, 1), (263, 4)):
+    expectations = [(None, 10**9, 4), (None, 576, 4), (None, 575, 3), (None, 472, 3), (None, 471, 4),  # two chunks: 208 blocks < 230 = 9/10 x 256
+                    (232, 471, 2), (233, 471, 4), (105, 368, 2), (105, 367, 1), (105, 264, 1), (105, 263, 4),
+                    (104, 10**9, 1)]                                                                   # (104: the root alone fills the machine)
+    for min_blocks, resident, chunks in expectations:
         out = join_kv_chunks(plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens,
                              plan.vnode_to_q_entries, plan.req_to_vnode_entries, plan.req_to_vnode_offs, plan.req_to_vnode_lens,
-                             plan.phase_node_nums, plan.phase_node_offsets, 4, 8, resident_blocks=resident)
-        assert out[7] == [25 * chunks + 30, 400], (resident, out[7])
+                             plan.phase_node_nums, plan.phase_node_offsets, 4, 8, min_blocks=min_blocks, resident_blocks=resident)
+        assert out[7] == [25 * chunks + 30, 400], (min_blocks, resident, out[7])
         assert set(out[6].tolist()) == {chunks + 2}
         root = sorted(set(zip(out[0][:25 * chunks].tolist(), out[1][:25 * chunks].tolist())))
         assert len(root) == chunks and root[0][0] == 0 and sum(n for _, n in root) == 4000
         assert all(a + n == b for (a, n), (b, _) in zip(root, root[1:])) and all(n % 64 == 0 for _, n in root[:-1])
-        new = _joined_plan(plan, 4, 8, None)
-        assert _attended(new, batch) == before
+    new = _joined_plan(plan, 4, 8, None)
+    assert _attended(new, batch) == before
+
+
+def test_many_equal_chains_are_not_cut_into_a_few_long_blocks():
+    """16 nodes of 1500 tokens under a 3000-token root that the planner merges into them: 16
+    runs of 4500 tokens in five chunks, 8 blocks per chunk -- 640 blocks.  No run covers the
+    machine by itself, so none is cut anew (one chunk of 4500 tokens for some of them would be
+    what the launch waits for)."""
+    from fasttree_hip.planner import FastTreeParams, fasttree_plan
+    tree, ptrs, batch = build_tree({"kind": "regular", "sizes": [1, 16, 256], "lens": [3000, 1500, 100]})
+    p = FastTreeParams(); p.set_values(0.66, 0.33, 0.1); p.set_q_tile_sizes([16, 4]); p.set_kv_tile_sizes([32, 32]); p.set_kv_group_num(4)
+    plan = fasttree_plan(tree, ptrs, batch, 8, [1024, 256], [256, 1024], [256, 256], p)
+    assert plan.phase_node_nums == [80, 256] and max(plan.vnode_to_kv_lens) == 1024
+    new = _joined_plan(plan, 4, 8, None)
+    assert new.phase_node_nums == [80, 256] and new.vnode_to_kv_lens == list(plan.vnode_to_kv_lens)
 
 
 def test_joining_kv_chunks_only_where_the_rows_fill_the_machine():
