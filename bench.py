@@ -61,9 +61,12 @@ WORKLOADS = {
 MEASURED_TRAFFIC = {("c3", "mi355x", "stage1"): 140.7e6, ("c4", "mi355x", "stage1"): 8715.3e6}
 
 PRESETS = {
-    "reference": dict(q_tiles=None, kv_tiles=(32, 32), kv_splits=(1024, 128), thr1=(132, 528), thr2=(132, 132)),
-    "mi355x": dict(q_tiles=None, kv_tiles=(32, 32), kv_splits=(1024, 256), thr1=(256, 1024), thr2=(256, 256)),
-    "wide": dict(q_tiles="wide", kv_tiles=(32, 32), kv_splits=(1024, 256), thr1=(256, 1024), thr2=(256, 256)),
+    "reference": dict(q_tiles=None, kv_tiles=(32, 32), kv_splits=(1024, 128), thr1=(132, 528), thr2=(132, 132),
+                      launch_order=False),
+    "mi355x": dict(q_tiles=None, kv_tiles=(32, 32), kv_splits=(1024, 256), thr1=(256, 1024), thr2=(256, 256),
+                   launch_order=True),
+    "wide": dict(q_tiles="wide", kv_tiles=(32, 32), kv_splits=(1024, 256), thr1=(256, 1024), thr2=(256, 256),
+                 launch_order=True),
 }
 
 
@@ -101,7 +104,8 @@ def build_problem(name, preset, device, seed=0):
     planner.VERBOSE = False
     t0 = time.perf_counter()
     aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, hq, hkv, 128, list(cfg["kv_splits"]), list(cfg["thr1"]),
-                                  list(cfg["thr2"]), params, device=device, kv_slot_map=inp.slot_map)
+                                  list(cfg["thr2"]), params, device=device, kv_slot_map=inp.slot_map,
+                                  launch_order=cfg.get("launch_order", True))
     plan_ms = (time.perf_counter() - t0) * 1e3
     elem = 2
     total = ptrs[-1]
@@ -171,7 +175,7 @@ def main():
     def step():
         fasttree_decode(inp.Q, inp.K_pool, inp.V_pool, o, *aux, prob["q_tiles"], prob["kv_tiles"], scale)
 
-    nums, offs = list(aux[11]), list(aux[12])
+    nums, offs = aux[11], aux[12]  # (the phase list carries the program table: passed as it is)
 
     def stage1():
         fasttree_decode_stage1(inp.Q, inp.K_pool, inp.V_pool, *aux[:6], scale, aux[9], aux[10], nums, offs,
@@ -286,7 +290,7 @@ def main():
         p2.set_kv_group_num(g)
         aux2, assign2 = fasttree_preparation(prob["tree"], inp.KV_ptrs, prob["batch"], prob["hq"], prob["hkv"], 128,
                                              [81920, 81920], [0, 0], [0, 0], p2, device=device,
-                                             kv_slot_map=inp.slot_map)
+                                             kv_slot_map=inp.slot_map, launch_order=True)
         om = torch.empty_like(inp.Q)
         ts = []
         for i in range(13):

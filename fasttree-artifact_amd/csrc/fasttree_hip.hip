@@ -133,6 +133,12 @@ struct Stage1Args {
   int wide_rows;                   // query rows the planner's tile gives a wide vnode (host hint for wide_chunks)
   int wide_chunks;                 // blocks per (wide vnode, kv head); block c serves row pieces c, c + wide_chunks, ..
   int block_slots;                 // blocks of the fused kernel the device runs at a time
+  // block programs written by the host (or null): four ints per program -- the wide vnodes
+  // [first, end) of the wide range, then first and count of its narrow vnodes in the narrow range
+  // (count < 0: they are served before the wide vnodes, else after them)
+  const int32_t* prog_table;
+  int num_programs;
+  int narrow_in_programs;          // narrow vnodes (from narrow_begin) that programs serve
   int g;
   int hkv;
   float scale_log2;  // sm_scale * log2(e)
@@ -465,7 +471,7 @@ __device__ __forceinline__ void merge_waves(float* xchg, WaveState<D, NQB>& st) 
 template <typename E, int D, int NQB, bool SPLIT_WAVES, bool GATHERED>
 __global__ void __launch_bounds__(kBlock) stage1_kernel(Stage1Args a) {
   using G = TileGeom<D>;
-  extern __shared__ __attribute__((aligned(16))) char smem[];
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int kvh = blockIdx.y;
   char* my_lds = smem + wave * G::kBytes;
@@ -500,26 +506,7 @@ __global__ void __launch_bounds__(kBlock) stage1_kernel(Stage1Args a) {
 // dependent chain, scores -> soft-max -> P.V; the matrix instructions of one wave overlap the
 // vector instructions of the other about half of the time.)
 // ---------------------------------------------------------------------------------------
-#ifdef FT_TIMING
-// Development aid, compiled out of the product: per-wave cycle counts of the wide kernel's
-// phases, written to a buffer set with ft_debug_set_timing().
-__device__ unsigned long long* g_timing = nullptr;
-__device__ int g_timing_steps = 0;  // 1: report per-step phases (scores, soft-max, P.V, steps) instead
-#define FT_CLOCK() __builtin_readcyclecounter()
-#define FT_TIME(...) __VA_ARGS__
-#else
-#define FT_TIME(...)
-#endif
-#ifndef FT_WIDE_WAVES
-#define FT_WIDE_WAVES 4
-#endif
-#ifndef FT_WIDE_BUFS
-#define FT_WIDE_BUFS 2
-#endif
-#ifndef FT_WIDE_IDX
-#define FT_WIDE_IDX 2048
-#endif
-constexpr int kWideWaves = FT_WIDE_WAVES;
+constexpr int kWideWaves = 4;
 constexpr int kWideBlock = kWave * kWideWaves;
 constexpr int kWideRows = 32 * kWideWaves;        // query rows one pass of a block serves
 constexpr int kWaveSlotsPerCu = 8;                // waves of these kernels a compute unit holds
@@ -536,7 +523,7 @@ template <int D> struct WideGeom {
   static constexpr int kChunks = D / 8;                  // 16-byte chunks per row
   static constexpr int kSub = 2;
   static constexpr int kTokens = kSub * kTileTokens;     // 64
-  static constexpr int kBufs = FT_WIDE_BUFS;
+  static constexpr int kBufs = 2;
   static constexpr int kAhead = kBufs - 1;               // super tiles in flight beyond the current one
   static constexpr int kTileBytes = kTileTokens * kRowBytes;
   static constexpr int kBytesK = kTokens * kRowBytes;
@@ -546,7 +533,7 @@ template <int D> struct WideGeom {
   static constexpr int kGroups = kTokens / kGroupRows;   // groups per matrix and super tile
   static constexpr int kUnits = 2 * kGroups / kWideWaves;                       // loads per wave and super tile
   static constexpr int kSlots = kGroups >= kWideWaves ? kGroups / kWideWaves : 1;  // distinct rows among them
-  static constexpr int kIdxCap = FT_WIDE_IDX;             // slot indices staged at a time (tokens)
+  static constexpr int kIdxCap = 2048;                    // slot indices staged at a time (tokens)
   static constexpr int kLds = kRing + 4 * kIdxCap;
   static __device__ __forceinline__ int swz(int row) { return (((row & 3) << 2) | ((row >> 2) & 3)) & (kChunks - 1); }
 };
@@ -596,8 +583,8 @@ __device__ __forceinline__ void load_q_frags32(const char* src, u32x4 (&qf)[D / 
 // Per-lane LDS byte addresses of the operand reads inside tile 0 of the current buffer, for
 // contraction step / dim block 0.  Thanks to the XOR layout the address for step ks (dim block
 // db) is the base with 32*ks (64*db) XOR-ed in; the second tile of the super tile is a constant
-// offset away and buffer b of the ring is b * kBytes further (the dynamic LDS segment starts
-// at 0).
+// offset away and buffer b of the ring is b * kBytes further (the ring starts on a multiple of the
+// row size).
 struct WideLane {
   unsigned k;     // K operand: row lane%32, chunk lane/32 (step ks: chunk 2*ks + lane/32)
   unsigned v_lo;  // transposed V read: tokens 4*(lane/32) + 0..3 (+16 for u = 1), dims 0..31
@@ -605,15 +592,20 @@ struct WideLane {
 };
 
 template <int D>
-__device__ __forceinline__ void init_lane(WideLane& la) {
+__device__ __forceinline__ void init_lane(WideLane& la, unsigned ring) {
   using W = WideGeom<D>;
   const int lane = threadIdx.x & 63;
   const int p32 = lane & 31, h = lane >> 5, p = lane & 15, gi = (lane >> 4) & 1;
-  la.k = p32 * W::kRowBytes + 16 * ((h & (W::kChunks - 1)) ^ W::swz(p32));
+  la.k = ring + p32 * W::kRowBytes + 16 * ((h & (W::kChunks - 1)) ^ W::swz(p32));
   const int row_lo = 4 * h + (p >> 2), row_hi = row_lo + 8;
   const int chunk = (2 * gi + ((p & 3) >> 1)) & (W::kChunks - 1);
-  la.v_lo = W::kBytesK + row_lo * W::kRowBytes + 16 * (chunk ^ W::swz(row_lo)) + 8 * (p & 1);
-  la.v_hi = W::kBytesK + row_hi * W::kRowBytes + 16 * (chunk ^ W::swz(row_hi)) + 8 * (p & 1);
+  la.v_lo = ring + W::kBytesK + row_lo * W::kRowBytes + 16 * (chunk ^ W::swz(row_lo)) + 8 * (p & 1);
+  la.v_hi = ring + W::kBytesK + row_hi * W::kRowBytes + 16 * (chunk ^ W::swz(row_hi)) + 8 * (p & 1);
+}
+
+// Byte offset of an object of the block's dynamic LDS segment within LDS.
+__device__ __forceinline__ unsigned lds_offset(const void* p) {
+  return (unsigned)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
 }
 
 __device__ __forceinline__ WideLane at_buffer(const WideLane& la0, unsigned buffer_offset) {
@@ -626,7 +618,8 @@ __device__ __forceinline__ WideLane at_buffer(const WideLane& la0, unsigned buff
 // in flight, which serialises the stream with the arithmetic.  Completion is awaited by hand
 // with wait_direct_loads<N>() before the block barrier that publishes a buffer.
 __device__ __forceinline__ void load_direct16(const char* src, unsigned lds_base) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_base) : "memory");
+  // (M0 holds the LDS address: bound as an operand, so the compiler writes it and knows it is live)
+  asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "{m0}"(lds_base) : "memory");
 }
 // Wait until at most N of this wave's vector-memory operations are still in flight (they finish
 // in order).
@@ -657,9 +650,8 @@ constexpr float kSlack = 8.f;
 // reads of 4 consecutive tokens each.  valid < 32 only on a run's last, partial tile.
 template <typename E, int D>
 __device__ __forceinline__ void tile_step32(const WideLane& la, unsigned off, int valid, float sc,
-                                            const u32x4 (&qf)[D / 16], WideState<D>& st FT_TIME(, unsigned long long* tt = nullptr)) {
+                                            const u32x4 (&qf)[D / 16], WideState<D>& st) {
   using W = WideGeom<D>;
-  FT_TIME(const unsigned long long tc0 = FT_CLOCK();)
   constexpr int KS = D / 16, DB = D / 32, NV = 2 * DB;
 
   // all K operands of the tile are requested before the first contraction needs one
@@ -683,7 +675,6 @@ __device__ __forceinline__ void tile_step32(const WideLane& la, unsigned off, in
     for (int j = 0; j < 16; ++j) s[j] = (8 * (j >> 2) + 4 * h + (j & 3) >= valid) ? -INFINITY : s[j];
   }
 
-  FT_TIME(__builtin_amdgcn_sched_barrier(0); const unsigned long long tc1 = FT_CLOCK(); __builtin_amdgcn_sched_barrier(0);)
   // the V^T operands do not depend on the probabilities: request them now, so that they arrive
   // under the soft-max arithmetic (they take the registers the K operands just left)
   const unsigned vlo = la.v_lo + off, vhi = la.v_hi + off;
@@ -726,10 +717,8 @@ __device__ __forceinline__ void tile_step32(const WideLane& la, unsigned off, in
 #pragma unroll
     for (int i = 0; i < 4; ++i) st.l = E::add_pair(pf[u][i], st.l);
 
-  FT_TIME(__builtin_amdgcn_sched_barrier(0); const unsigned long long tc2 = FT_CLOCK(); __builtin_amdgcn_sched_barrier(0);)
 #pragma unroll
   for (int i = 0; i < NV; ++i) st.o[i % DB] = E::mfma32(vf[i], pf[i / DB], st.o[i % DB]);
-  FT_TIME(if (tt) { __builtin_amdgcn_sched_barrier(0); const unsigned long long tc3 = FT_CLOCK(); tt[0] += tc1 - tc0; tt[1] += tc2 - tc1; tt[2] += tc3 - tc2; tt[3] += 1; })
 }
 
 template <int D>
@@ -795,7 +784,8 @@ __device__ __forceinline__ void merge_token_groups(float* xchg, WideState<D>& st
   }
 }
 
-// One block (kWideWaves waves) per (vnode, kv head, chunk of kWideRows query rows).  The block
+// One block (kWideWaves waves) serves the row pieces chunk, chunk + chunks, ... (kWideRows query
+// rows each) of a vnode for one kv head.  The block
 // streams the vnode's KV run through a ring of kBufs 64-token LDS buffers with direct
 // global->LDS loads, kBufs - 1 super tiles ahead of the one being consumed; the run's slot
 // indices are staged in LDS first so that nothing but those loads is in flight in the loop.
@@ -803,11 +793,10 @@ __device__ __forceinline__ void merge_token_groups(float* xchg, WideState<D>& st
 // (RG * TG = kWideWaves): a wave consumes the 32-token tiles t with t % TG == tg for the rows of
 // its row group, and the TG states of a row group are merged at the end.
 template <typename E, int D, bool GATHERED>
-__device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int local_vnode, const VnodeView& vn,
-                                           int kvh, int chunk) {
+__device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, const VnodeView& vn, int kvh, int chunk,
+                                           int chunks) {
   using W = WideGeom<D>;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  FT_TIME(const unsigned long long rt_entry = wall_clock64();)
   const int rows_total = vn.q_len * a.g;
   const int nsuper = (vn.kv_len + W::kTokens - 1) / W::kTokens;
 
@@ -817,9 +806,10 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
   const char* vbase = a.v + 2 * ((int64_t)kvh * a.sv1);
   const unsigned k_stride = (unsigned)(2 * a.sk0), v_stride = (unsigned)(2 * a.sv0);  // bytes, < 2^32 (checked by the host)
   int* idx_lds = reinterpret_cast<int*>(smem + W::kRing);
+  const unsigned ring = lds_offset(smem);
 
-  // this block's pieces of kWideRows rows: chunk, chunk + wide_chunks, ...
-  for (int piece = chunk; piece * kWideRows < rows_total; piece += a.wide_chunks) {
+  // this block's pieces of kWideRows rows: chunk, chunk + chunks, ...
+  for (int piece = chunk; piece * kWideRows < rows_total; piece += chunks) {
   const int rows_end = min((piece + 1) * kWideRows, rows_total);
   for (int row0 = piece * kWideRows; row0 < rows_end;) {
     // waves as rgroups row groups x tgroups token groups: halve the row groups (down to a token
@@ -840,7 +830,7 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
     WideState<D> st;
     reset_state<D>(st);
     WideLane la0;
-    init_lane<D>(la0);
+    init_lane<D>(la0, ring);
     unsigned cur = 0;  // byte offset of the ring buffer that holds the current super tile
 
     // slot indices of tokens [idx_base, idx_base + kIdxCap) of the run, staged by the whole block
@@ -868,7 +858,7 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
           stage_indices(idx_base + W::kIdxCap);
         }
       }
-      const unsigned buf = (unsigned)(j % W::kBufs) * W::kBytes;
+      const unsigned buf = ring + (unsigned)(j % W::kBufs) * W::kBytes;
       unsigned srow[W::kSlots];
       unsigned chunk[W::kSlots];
 #pragma unroll
@@ -899,20 +889,15 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
     // (and the compiler must see the fragments as complete, or it keeps a wait for them in the loop)
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(qf[ks]));
-    FT_TIME(unsigned long long t_start = FT_CLOCK(); unsigned long long rt_start = wall_clock64(); unsigned long long t_wait = 0, t_bar = 0, t_issue = 0, t_comp = 0; unsigned long long t_step[4] = {0, 0, 0, 0};)
     for (int super = 0; super < nsuper; ++super) {
       // publish super tile `super` to the block; the ones after it may stay in flight
-      FT_TIME(unsigned long long c0 = FT_CLOCK();)
       const int behind = min(nsuper - 1 - super, W::kAhead - 1);
       if (behind >= 2) wait_direct_loads<2 * W::kUnits>();
       else if (behind == 1) wait_direct_loads<W::kUnits>();
       else wait_direct_loads<0>();
-      FT_TIME(unsigned long long c1 = FT_CLOCK();)
       __syncthreads();
-      FT_TIME(unsigned long long c2 = FT_CLOCK();)
       // the buffer consumed before that barrier is free: refill it
       issue_rows(super + W::kAhead);
-      FT_TIME(unsigned long long c3 = FT_CLOCK();)
       if (active) {
         const WideLane la = at_buffer(la0, cur);
 #pragma unroll 1
@@ -920,17 +905,11 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, int 
           const int tile = super * W::kSub + sub;
           if ((tile & (tgroups - 1)) != tg) continue;
           const int valid = vn.kv_len - tile * kTileTokens;
-          if (valid > 0) tile_step32<E, D>(la, sub * W::kTileBytes, valid, a.scale_log2, qf, st FT_TIME(, t_step));
+          if (valid > 0) tile_step32<E, D>(la, sub * W::kTileBytes, valid, a.scale_log2, qf, st);
         }
       }
       cur = cur + W::kBytes == W::kRing ? 0u : cur + W::kBytes;
-      FT_TIME(unsigned long long c4 = FT_CLOCK(); t_wait += c1 - c0; t_bar += c2 - c1; t_issue += c3 - c2; t_comp += c4 - c3;)
     }
-    FT_TIME(if (g_timing && lane == 0) {
-      unsigned long long* out = g_timing + ((size_t)blockIdx.x * kWideWaves + wave) * 8;
-      out[0] = g_timing_steps ? t_step[0] : t_wait; out[1] = g_timing_steps ? t_step[1] : t_bar; out[2] = g_timing_steps ? t_step[2] : t_issue; if (g_timing_steps != 2) out[3] = g_timing_steps ? t_step[3] : t_comp; out[4] = g_timing_steps == 2 ? rt_entry : FT_CLOCK() - t_start; out[5] = nsuper + 1000 * local_vnode + 100000 * chunk;
-      out[6] = rt_start; out[7] = wall_clock64();
-    })
     finish_state<D>(st);
     if (tgroups > 1) merge_token_groups<D>(reinterpret_cast<float*>(smem), st, rg, tg, tgroups, active);
     if (active && tg == 0) write_partials32<D>(a, vn, kvh, my_row0, st);
@@ -972,6 +951,7 @@ __device__ __forceinline__ void narrow_attend(const Stage1Args& a, const VnodeVi
   const int p = lane & 15, c = lane >> 4;
   const int ntiles = (vn.kv_len + kTileTokens - 1) / kTileTokens;
   int* idx_lds = reinterpret_cast<int*>(smem + lds0 + N::kBytes);
+  const unsigned tile0_addr = lds_offset(smem) + lds0;  // the wave's K tile; its V tile follows
 
   // loader role: 16-byte slot `pos` of row `grp_row` in each 1 KB group
   const int grp_row = lane / N::kChunks, pos = lane % N::kChunks;
@@ -985,8 +965,8 @@ __device__ __forceinline__ void narrow_attend(const Stage1Args& a, const VnodeVi
 #pragma unroll
   for (int tb = 0; tb < 2; ++tb) {
     const int kr = 16 * tb + p, vr = 16 * tb + 4 * c + (p >> 2);
-    k_addr[tb] = lds0 + kr * N::kRowBytes + 16 * ((c & (N::kChunks - 1)) ^ N::swz(kr));
-    v_addr[tb] = lds0 + N::kBytesK + vr * N::kRowBytes + 16 * ((((p & 3) >> 1) & (N::kChunks - 1)) ^ N::swz(vr)) + 8 * (p & 1);
+    k_addr[tb] = tile0_addr + kr * N::kRowBytes + 16 * ((c & (N::kChunks - 1)) ^ N::swz(kr));
+    v_addr[tb] = tile0_addr + N::kBytesK + vr * N::kRowBytes + 16 * ((((p & 3) >> 1) & (N::kChunks - 1)) ^ N::swz(vr)) + 8 * (p & 1);
   }
 
   // start-up chain: [request id of the lane's row, slot indices] -> [Q fragments, first K/V rows].
@@ -1034,7 +1014,7 @@ __device__ __forceinline__ void narrow_attend(const Stage1Args& a, const VnodeVi
       for (int g = 0; g < N::kGroups; ++g) {
         const int row = g * N::kGroupRows + grp_row;
         const char* src = (is_v ? vbase : kbase) + (uint64_t)srow[g] * (is_v ? v_stride : k_stride) + 16 * (pos ^ N::swz(row));
-        load_direct16(src, lds0 + (is_v ? N::kBytesK : 0) + g * 1024);
+        load_direct16(src, tile0_addr + (is_v ? N::kBytesK : 0) + g * 1024);
       }
     };
     stage_indices(tile0 * kTileTokens);
@@ -1164,7 +1144,7 @@ template <typename E, int D, bool GATHERED>
 __device__ __forceinline__ void narrow_item(const Stage1Args& a, char* smem, int slot, int share, bool exists,
                                             int vnode, int kvh) {
   using N = NarrowGeom<D>;
-  const unsigned lds0 = (unsigned)slot * N::kLds;  // the dynamic LDS segment starts at 0
+  const unsigned lds0 = (unsigned)slot * N::kLds;  // byte offset of the wave's area in the block's LDS segment
   VnodeView vn{0, 0, 0, 0};
   if (exists) vn = load_vnode<GATHERED>(a, vnode);
   const int rows_total = vn.q_len * a.g;
@@ -1202,7 +1182,7 @@ __device__ __forceinline__ void narrow_item(const Stage1Args& a, char* smem, int
 // these latency-bound waves share a compute unit.
 template <typename E, int D, bool GATHERED>
 __global__ void __launch_bounds__(kWideBlock) stage1_narrow_kernel(Stage1Args a) {
-  extern __shared__ __attribute__((aligned(16))) char smem[];
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int local_vnode = blockIdx.x / a.hkv;
   narrow_item<E, D, GATHERED>(a, smem, wave, a.narrow_share, true, a.narrow_begin + local_vnode,
@@ -1227,8 +1207,8 @@ __device__ __forceinline__ int wide_vnode_of_rank(const Stage1Args& a, char* sme
     view = load_vnode<GATHERED>(a, a.vnode_begin + target);
     return target;
   }
-  // keys[u]: work of vnode u in 24 bits (a float's exponent and leading mantissa bits), then
-  // 255 - u: larger key = earlier, no two equal; 0 for a vnode that is not the head of a group
+  // keys[u]: work of vnode u in 23 bits (a float's exponent and leading mantissa bits), then
+  // 256 - u: larger key = earlier, no two equal; 0 for a vnode that is not the head of a group
   unsigned* keys = reinterpret_cast<unsigned*>(smem);
   VnodeView* views = reinterpret_cast<VnodeView*>(keys + kMaxRanked);
   int* group_q_len = reinterpret_cast<int*>(views + kMaxRanked);
@@ -1279,7 +1259,9 @@ __device__ __forceinline__ int wide_vnode_of_rank(const Stage1Args& a, char* sme
       const VnodeView& tail = views[min(last, head + m - 1)];
       q_len = tail.q_off + tail.q_len - views[tid].q_off;
       const float work = (float)q_len * (float)a.g * (float)views[tid].kv_len;
-      mine = ((__builtin_bit_cast(unsigned, work) >> 7) << 8) | (unsigned)(255 - tid);
+      // (256 - tid is never 0: the key of a vnode without work must not be the 0 of "no group")
+      static_assert(kMaxRanked <= 256, "the low nine bits of a key hold 256 - tid");
+      mine = ((__builtin_bit_cast(unsigned, work) >> 8) << 9) | (unsigned)(256 - tid);
     }
     group_q_len[tid] = q_len;
   }
@@ -1316,12 +1298,35 @@ __device__ __forceinline__ int wide_vnode_of_rank(const Stage1Args& a, char* sme
 // blocks follow and fill the machine while the wide blocks drain.
 template <typename E, int D, bool GATHERED>
 __global__ void __launch_bounds__(kWideBlock, 512 / kWideBlock) stage1_fused_kernel(Stage1Args a) {
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  FT_TIME(if (g_timing && g_timing_steps == 2 && (threadIdx.x & 63) == 0) g_timing[((size_t)blockIdx.x * kWideWaves + (threadIdx.x >> 6)) * 8 + 3] = wall_clock64();)
-  const int wide_blocks = a.vnode_count * a.wide_chunks * a.hkv;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int wide_blocks = a.prog_table ? a.num_programs * a.hkv : a.vnode_count * a.wide_chunks * a.hkv;
   const int wide_index = blockIdx.x, narrow_index = (int)blockIdx.x - wide_blocks;
   const bool is_wide = (int)blockIdx.x < wide_blocks;
-  if (is_wide) {
+  if (is_wide && a.prog_table) {
+    // A block program written by the host, for one kv head (kv head fastest: the eight blocks of
+    // a program land on the eight XCDs, and a head's K/V only ever enters one XCD's L2): its wide
+    // vnodes one after the other, and its narrow vnodes, one wave each, before or after them.
+    // Of the two blocks that share a compute unit one starts with its narrow vnodes and the
+    // other ends with them, so that the memory-bound narrow vnodes of one run under the
+    // arithmetic-bound wide vnodes of the other.
+    const int program = wide_index / a.hkv;
+    const int kvh = wide_index - program * a.hkv;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wide_first = a.prog_table[4 * program], wide_end = a.prog_table[4 * program + 1];
+    const int narrow_first = a.prog_table[4 * program + 2], narrow_signed = a.prog_table[4 * program + 3];
+    const int narrow_count = narrow_signed < 0 ? -narrow_signed : narrow_signed;
+    auto narrow_vnodes = [&]() {
+      for (int i = wave; i < narrow_count; i += kWideWaves)
+        narrow_item<E, D, GATHERED>(a, smem, wave, 1, true, a.narrow_begin + narrow_first + i, kvh);
+      __syncthreads();  // the waves' tiles become the ring of the next wide vnode
+    };
+    if (narrow_signed < 0) narrow_vnodes();
+    for (int v = wide_first; v < wide_end; ++v) {
+      const VnodeView vn = load_vnode<GATHERED>(a, a.vnode_begin + v);
+      wide_block<E, D, GATHERED>(a, smem, vn, kvh, 0, 1);
+    }
+    if (narrow_signed > 0) narrow_vnodes();
+  } else if (is_wide) {
     const int per_rank = a.wide_chunks * a.hkv;
     const int rank = wide_index / per_rank;
     const int rest = wide_index - rank * per_rank;
@@ -1332,22 +1337,17 @@ __global__ void __launch_bounds__(kWideBlock, 512 / kWideBlock) stage1_fused_ker
     const int slot = rest / a.hkv;
     const int chunk = (slot + (rank >> 1)) % a.wide_chunks;
     VnodeView vn;
-    const int local_vnode = wide_vnode_of_rank<GATHERED>(a, smem, rank, vn);
-    wide_block<E, D, GATHERED>(a, smem, local_vnode, vn, rest - slot * a.hkv, chunk);
+    (void)wide_vnode_of_rank<GATHERED>(a, smem, rank, vn);
+    wide_block<E, D, GATHERED>(a, smem, vn, rest - slot * a.hkv, chunk, a.wide_chunks);
   } else {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int share = a.narrow_share;
-    const int item = narrow_index * (kWideWaves / share) + wave / share;
+    const int item = narrow_index * (kWideWaves / share) + wave / share + a.narrow_in_programs * a.hkv;
     const bool exists = item < a.narrow_count * a.hkv;
     if (share == 1 && !exists) return;  // whole wave; no block barrier below in this mode
     const int local_vnode = item / a.hkv;
     const int kvh = item - local_vnode * a.hkv;
-    FT_TIME(unsigned long long t_start = FT_CLOCK(); unsigned long long rt_start = wall_clock64();)
     narrow_item<E, D, GATHERED>(a, smem, wave, share, exists, a.narrow_begin + local_vnode, kvh);
-    FT_TIME(if (g_timing && (threadIdx.x & 63) == 0) {
-      unsigned long long* out = g_timing + ((size_t)blockIdx.x * kWideWaves + wave) * 8;
-      out[4] = FT_CLOCK() - t_start; out[5] = 0; out[6] = rt_start; out[7] = wall_clock64();
-    })
   }
 }
 
@@ -1540,13 +1540,14 @@ int launch_stage1_fused(const Stage1Args& a0, hipStream_t stream) {
     configured = true;
   }
   Stage1Args a = a0;
-  const int64_t narrow_items = (int64_t)a.narrow_count * a.hkv;
+  const int64_t narrow_items = (int64_t)(a.narrow_count - a.narrow_in_programs) * a.hkv;  // those of the trailing blocks
   a.narrow_share = narrow_share_for(narrow_items);
   const int per_block = kWideWaves / a.narrow_share;
   const int64_t narrow_blocks = (narrow_items + per_block - 1) / per_block;
   a.wide_chunks = std::max(1, std::min(8, (a.wide_rows + kWideRows - 1) / kWideRows));
   a.block_slots = wave_slots() / kWideWaves;
-  const int64_t blocks = (int64_t)a.vnode_count * a.wide_chunks * a.hkv + narrow_blocks;
+  const int64_t wide_blocks = a.prog_table ? (int64_t)a.num_programs * a.hkv : (int64_t)a.vnode_count * a.wide_chunks * a.hkv;
+  const int64_t blocks = wide_blocks + narrow_blocks;
   if (blocks == 0) return FT_OK;
   if (blocks > INT32_MAX) return FT_ERR_ARGUMENT;
   hipLaunchKernelGGL(kern, dim3((unsigned)blocks, 1, 1), dim3(kWideBlock, 1, 1), lds, stream, a);
@@ -1592,7 +1593,7 @@ int launch_stage1_d(const Stage1Args& a, hipStream_t stream) {
     }
     return FT_OK;
   } else {
-    if (a.vnode_count == 0) return launch_stage1_narrow<E, D, GATHERED>(a, stream);
+    if (a.vnode_count == 0 && !a.prog_table) return launch_stage1_narrow<E, D, GATHERED>(a, stream);
     return launch_stage1_fused<E, D, GATHERED>(a, stream);
   }
 }
@@ -1644,15 +1645,6 @@ int check_common(int d, int g, int dtype) {
 }
 
 }  // namespace
-
-#ifdef FT_TIMING
-extern "C" int ft_debug_set_timing(unsigned long long* buf) {
-  return hipMemcpyToSymbol(HIP_SYMBOL(g_timing), &buf, sizeof(buf)) == hipSuccess ? 0 : -1;
-}
-extern "C" int ft_debug_set_timing_steps(int on) {
-  return hipMemcpyToSymbol(HIP_SYMBOL(g_timing_steps), &on, sizeof(on)) == hipSuccess ? 0 : -1;
-}
-#endif
 
 extern "C" {
 
@@ -1808,6 +1800,62 @@ int ft_stage1_phases(const void* q, const void* k, const void* v,
   for (int phase = 0; phase < 2; ++phase)
     if (pending[phase]) assign(a, narrow[phase], phase_node_offsets[phase], phase_node_nums[phase]);
   return launch_stage1<false>(a, head_dim, dtype, stream);
+}
+
+int ft_stage1_programs(const void* q, const void* k, const void* v,
+                       int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+                       const int32_t* vnode_to_kv_entries, const int32_t* vnode_to_kv_offs,
+                       const int32_t* vnode_to_kv_lens, const int32_t* vnode_to_q_entries,
+                       const int32_t* vnode_to_q_offs, const int32_t* vnode_to_q_lens,
+                       float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
+                       const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
+                       const int32_t* prog_table, int num_programs, int narrow_in_programs,
+                       int num_qo_heads, int num_kv_heads, int head_dim,
+                       float sm_scale, int dtype, ft_stream_t stream) {
+  if (!phase_node_nums || !phase_node_offsets) return FT_ERR_NULL_POINTER;
+  if (num_kv_heads < 1 || num_qo_heads % num_kv_heads != 0) return FT_ERR_GROUP;
+  const int g = num_qo_heads / num_kv_heads;
+  if (int rc = check_common(head_dim, g, dtype)) return rc;
+  if (head_dim > 128) return FT_ERR_HEAD_DIM;  // the program table is for the direct-load kernels
+  if (phase_node_nums[0] == 0 && phase_node_nums[1] == 0) return FT_OK;
+  Stage1Args a;
+  if (int rc = stage1_setup(a, q, k, v, sq0, sq1, sk0, sk1, sv0, sv1, vnode_to_kv_entries, vnode_to_kv_offs,
+                            vnode_to_kv_lens, vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, num_kv_heads, g,
+                            head_dim, sm_scale, mid_o, so0, so1, mid_lse, sl0, dtype))
+    return rc;
+  for (int phase = 0; phase < 2; ++phase)
+    if (!range_ok(phase_node_offsets[phase], phase_node_nums[phase], num_kv_heads)) return FT_ERR_ARGUMENT;
+  if (num_programs < 0 || (int64_t)num_programs * num_kv_heads > INT32_MAX) return FT_ERR_ARGUMENT;
+  if (num_programs > 0 && !prog_table) return FT_ERR_NULL_POINTER;
+  if (narrow_in_programs < 0 || narrow_in_programs > phase_node_nums[1]) return FT_ERR_ARGUMENT;
+  if (num_programs == 0 && (phase_node_nums[0] > 0 || narrow_in_programs > 0)) return FT_ERR_ARGUMENT;
+  a.vnode_begin = phase_node_offsets[0]; a.vnode_count = phase_node_nums[0];
+  a.narrow_begin = phase_node_offsets[1]; a.narrow_count = phase_node_nums[1];
+  if (num_programs > 0) { a.prog_table = prog_table; a.num_programs = num_programs; a.narrow_in_programs = narrow_in_programs; }
+  a.wide_rows = kWideRows;
+  return launch_stage1<false>(a, head_dim, dtype, stream);
+}
+
+int ft_decode_programs(const void* q, const void* k, const void* v, void* o,
+                       int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+                       int64_t oo0, int64_t oo1,
+                       const int32_t* vnode_to_kv_entries, const int32_t* vnode_to_kv_offs,
+                       const int32_t* vnode_to_kv_lens, const int32_t* vnode_to_q_entries,
+                       const int32_t* vnode_to_q_offs, const int32_t* vnode_to_q_lens,
+                       const int32_t* req_to_vnode_entries, const int32_t* req_to_vnode_offs,
+                       const int32_t* req_to_vnode_lens,
+                       float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
+                       const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
+                       const int32_t* prog_table, int num_programs, int narrow_in_programs,
+                       int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
+                       float sm_scale, int dtype, ft_stream_t stream) {
+  if (int rc = ft_stage1_programs(q, k, v, sq0, sq1, sk0, sk1, sv0, sv1, vnode_to_kv_entries, vnode_to_kv_offs,
+                                  vnode_to_kv_lens, vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, mid_o, so0,
+                                  so1, mid_lse, sl0, phase_node_nums, phase_node_offsets, prog_table, num_programs,
+                                  narrow_in_programs, num_qo_heads, num_kv_heads, head_dim, sm_scale, dtype, stream))
+    return rc;
+  return ft_stage2(req_to_vnode_entries, req_to_vnode_offs, req_to_vnode_lens, mid_o, so0, so1, mid_lse, sl0, o, oo0,
+                   oo1, batch_size, num_qo_heads, head_dim, dtype, stream);
 }
 
 int ft_decode(const void* q, const void* k, const void* v, void* o,

@@ -10,15 +10,15 @@ from .kv_tree import (  # noqa: F401
     nodes_from_rows, assign_requests, kv_prefix_sums,
 )
 from .planner import (  # noqa: F401
-    FastTreeParams, FastTreePlan, PlanBuffers, fasttree_plan, fasttree_preparation, join_kv_chunks, vnodes_in_launch_order,
-    _tree_heuristic,
+    FastTreeParams, FastTreePlan, PlanBuffers, fasttree_plan, fasttree_preparation, _tree_heuristic,
 )
+from .launch_schedule import LaunchPhases, LaunchSchedule, block_programs  # noqa: F401
 
 __all__ = [
     "KVTreeNode", "retrive_from_file", "generate_tree", "generate_irregular_tree", "save_tree",
     "nodes_from_rows", "assign_requests", "kv_prefix_sums",
-    "FastTreeParams", "FastTreePlan", "PlanBuffers", "fasttree_plan", "fasttree_preparation", "join_kv_chunks",
-    "vnodes_in_launch_order",
+    "FastTreeParams", "FastTreePlan", "PlanBuffers", "fasttree_plan", "fasttree_preparation",
+    "LaunchPhases", "LaunchSchedule", "block_programs",
     "fasttree_decode",
 ]
 

@@ -67,6 +67,24 @@ def fasttree_decode(
     if mid_o.dtype != torch.float32 or mid_lse.dtype != torch.float32:
         raise _lib.FastTreeLibraryError("mid_o and mid_lse must be float32")
     lib = _lib.load()
+    programs = getattr(phase_node_nums, "prog_table", None)
+    if programs is not None and q.shape[-1] <= 128:
+        # the launch was arranged as block programs (launch_schedule.block_programs)
+        rc = lib.ft_decode_programs(
+            q.data_ptr(), k_buffer.data_ptr(), v_buffer.data_ptr(), o.data_ptr(),
+            q.stride(0), q.stride(1), k_buffer.stride(0), k_buffer.stride(1),
+            v_buffer.stride(0), v_buffer.stride(1), o.stride(0), o.stride(1),
+            vnode_to_kv_entries.data_ptr(), vnode_to_kv_offs.data_ptr(), vnode_to_kv_lens.data_ptr(),
+            vnode_to_q_entries.data_ptr(), vnode_to_q_offs.data_ptr(), vnode_to_q_lens.data_ptr(),
+            req_to_vnode_entries.data_ptr(), req_to_vnode_offs.data_ptr(), req_to_vnode_lens.data_ptr(),
+            mid_o.data_ptr(), mid_o.stride(0), mid_o.stride(1), mid_lse.data_ptr(), mid_lse.stride(0),
+            _lib.int32_pair(phase_node_nums), _lib.int32_pair(phase_node_offsets),
+            programs.data_ptr(), int(phase_node_nums.num_programs), int(phase_node_nums.narrow_in_programs),
+            q.shape[0], q.shape[1], k_buffer.shape[1], q.shape[-1],
+            float(sm_scale), _dtype_code(q), _stream_handle(q),
+        )
+        _lib.check(rc, "ft_decode_programs")
+        return
     rc = lib.ft_decode(
         q.data_ptr(), k_buffer.data_ptr(), v_buffer.data_ptr(), o.data_ptr(),
         q.stride(0), q.stride(1), k_buffer.stride(0), k_buffer.stride(1),
@@ -90,6 +108,20 @@ def fasttree_decode_stage1(q, k_buffer, v_buffer, vnode_to_kv_entries, vnode_to_
     (the role of _fasttree_decode_stage1, kernel_bench/fasttree.py:416-479)."""
     _need_gpu(q, k_buffer, v_buffer, mid_o, mid_lse)
     lib = _lib.load()
+    programs = getattr(phase_node_nums, "prog_table", None)
+    if programs is not None and q.shape[-1] <= 128:
+        rc = lib.ft_stage1_programs(
+            q.data_ptr(), k_buffer.data_ptr(), v_buffer.data_ptr(),
+            q.stride(0), q.stride(1), k_buffer.stride(0), k_buffer.stride(1), v_buffer.stride(0), v_buffer.stride(1),
+            vnode_to_kv_entries.data_ptr(), vnode_to_kv_offs.data_ptr(), vnode_to_kv_lens.data_ptr(),
+            vnode_to_q_entries.data_ptr(), vnode_to_q_offs.data_ptr(), vnode_to_q_lens.data_ptr(),
+            mid_o.data_ptr(), mid_o.stride(0), mid_o.stride(1), mid_lse.data_ptr(), mid_lse.stride(0),
+            _lib.int32_pair(phase_node_nums), _lib.int32_pair(phase_node_offsets),
+            programs.data_ptr(), int(phase_node_nums.num_programs), int(phase_node_nums.narrow_in_programs),
+            q.shape[1], k_buffer.shape[1], q.shape[-1], float(sm_scale), _dtype_code(q), _stream_handle(q),
+        )
+        _lib.check(rc, "ft_stage1_programs")
+        return
     rc = lib.ft_stage1_phases(
         q.data_ptr(), k_buffer.data_ptr(), v_buffer.data_ptr(),
         q.stride(0), q.stride(1), k_buffer.stride(0), k_buffer.stride(1), v_buffer.stride(0), v_buffer.stride(1),

@@ -1,0 +1,432 @@
+"""Launch schedule of the first decode stage on an MI355X: the planner's vnodes re-cut into
+equal-work block programs.
+
+The reference launches one thread block per (vnode, KV head) and leaves the order and the
+placement to the hardware dispatcher (kernel_bench/fasttree.py:443-479, grid = (node_num,
+head_num)).  On a part with 256 compute units a launch of a few hundred blocks of unequal
+length ends when its most loaded compute unit does: with the planner's fixed KV split the
+3-level tree of the headline benchmark puts 1.5 times the average work on some units.  The
+functions here take the planner's lists (in the reference's order, kernel_bench/fasttree.py:
+193-262) and return lists that describe the same computation -- every request still attends
+every token of its root path exactly once, each (request, piece) pair through one scratch row
+that the second stage merges -- arranged for the machine:
+
+* The wide vnodes (more than 16 query rows) over one KV run are undone: the planner's KV chunks
+  of a node are joined back into the node's run and its query tiles into the node's request
+  list.  The run is then cut anew into row chunks of ``block_rows`` query rows (what one block
+  of the kernel serves per pass) and, along the tokens, wherever a block program is full.
+* A *block program* is a list of consecutive vnodes that one thread block serves, one after the
+  other, for one KV head.  Programs hold equal work (tile steps plus a start-up charge per
+  vnode); there are ``block_slots // num_kv_heads`` of them per round and head, so that one
+  round of programs fills every compute unit exactly once and all of them end together.
+* Narrow vnodes (at most 16 query rows) keep the planner's chunks and are served one wave each.
+  When the programs fill the machine there is no room for blocks of their own beside them, so
+  they are dealt to the programs, longest first, in equal shares: a program serves its narrow
+  vnodes with its four waves before its wide vnodes or after them.  The two blocks that share a
+  compute unit get opposite orders, so the memory round trips of one block's narrow vnodes are
+  filled by the matrix work of the other.  Narrow vnodes that would take a program longer than
+  its wide vnodes stay in blocks of their own after the programs.
+
+Nothing refers to a vnode by its position (the per-request lists name scratch rows), and the
+kernels compute a vnode of any number of rows and tokens, so the arrangement changes the
+schedule, not the result.  The lists this module returns are a complete plan on their own:
+``fasttree_decode`` gives the same result with or without the program table.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List
+
+import numpy as np
+
+#: Query rows one block of the first-stage kernel serves per pass (4 waves x 32 rows).
+BLOCK_ROWS = 128
+#: Blocks of the first-stage kernel an MI355X runs at a time (two per compute unit).
+BLOCK_SLOTS = 512
+#: KV tokens of one tile step.
+TILE_TOKENS = 32
+#: Start-up and wind-down of one vnode inside a program, in tile steps (three dependent memory
+#: round trips before the first step, the partial results after the last: about 6 us measured,
+#: against 1.2 us per step of a block that shares its compute unit).
+VNODE_STARTUP_TILES = 5.0
+#: A narrow vnode on one wave, in the same unit: its start-up and one 32-token step.
+NARROW_STARTUP_TILES = 3.8
+NARROW_STEP_TILES = 0.85
+#: Microseconds per tile step of a block that shares its compute unit with another wide block,
+#: and of one that does not (measured on the 3-level tree of the headline benchmark).
+TILE_US_SHARED = 1.19
+TILE_US_ALONE = 0.95
+#: Bytes per microsecond the narrow vnodes stream at most (rows of 2 * head_dim bytes at random slots).
+NARROW_BYTES_PER_US = 5.6e6
+#: Waves the machine holds (narrow vnodes in flight).
+WAVE_SLOTS = 2048
+#: Waves of a block (each serves one narrow vnode at a time).
+BLOCK_WAVES = 4
+#: A launch is cut into equal programs only if every program gets at least this much work
+#: (tile steps); smaller launches keep the planner's chunks, one vnode per program.
+MIN_PROGRAM_TILES = 12.0
+#: Most work (tile steps) one program may hold; larger launches run several rounds of programs.
+MAX_PROGRAM_TILES = 160.0
+#: Pieces are cut at multiples of this many tokens (two tiles: one trip of the kernel's loop) and
+#: are not made shorter than MIN_PIECE_TOKENS.
+CUT_TOKENS = 64
+MIN_PIECE_TOKENS = 128
+#: A wide run of at most LIGHT_ROWS query rows and LIGHT_WORK query rows x KV tokens is served
+#: with the narrow vnodes when the launch has more wide blocks than the machine runs at a time
+#: (short runs under a few dozen rows are bound by memory latency, and the narrow path has eight
+#: of them in flight per compute unit).
+LIGHT_WORK = 4096
+LIGHT_ROWS = 64
+NARROW_ROWS = 16
+
+
+class LaunchPhases(list):
+    """``phase_node_nums`` as the decode call takes it (a list of two counts) that also carries
+    the block programs of the launch: ``prog_table`` (int32 device tensor, four entries per
+    program: first and end of its wide vnodes within the first phase, first and signed count of
+    its narrow vnodes within the second; a negative count: served before the wide ones) or None,
+    ``num_programs`` and ``narrow_in_programs`` (how many vnodes at the head of the second phase
+    belong to programs)."""
+
+    prog_table = None
+    num_programs = 0
+    narrow_in_programs = 0
+
+
+@dataclass
+class LaunchSchedule:
+    kv_offs: np.ndarray
+    kv_lens: np.ndarray
+    q_offs: np.ndarray
+    q_lens: np.ndarray
+    q_entries: np.ndarray        # request of every scratch row
+    req_entries: np.ndarray      # scratch rows per request, back to back, then 32 x -1
+    req_offs: np.ndarray
+    req_lens: np.ndarray
+    phase_node_nums: List[int]
+    phase_node_offsets: List[int]
+    prog_table: np.ndarray       # (num_programs, 4); see LaunchPhases
+    narrow_in_programs: int
+    program_tiles: np.ndarray    # modelled work of every program (for tests and reports)
+    block_slots: int = BLOCK_SLOTS
+    modelled_us: float = 0.0     # modelled duration of the launch
+
+    @property
+    def num_rows(self) -> int:
+        return int(len(self.q_entries))
+
+    @property
+    def num_programs(self) -> int:
+        return int(self.prog_table.shape[0])
+
+
+def _tile_weight(rows: int) -> float:
+    """Share of a block's time one tile step of a piece with ``rows`` query rows takes: the
+    block's four waves form row groups of 32 rows; with half of them idle they split the tokens
+    of a 64-token super tile instead (two ways: a super tile holds two tile steps)."""
+    return 1.0 if rows > 64 else 0.55
+
+
+def _row_chunks(n_requests: int, cap: int):
+    """``n_requests`` cut into the fewest chunks of at most ``cap``, as even as possible (a last
+    chunk of a few rows would leave most of a block's waves without rows)."""
+    count = max(1, -(-n_requests // cap))
+    base, extra = divmod(n_requests, count)
+    lo = 0
+    for i in range(count):
+        size = base + (1 if i < extra else 0)
+        yield lo, lo + size
+        lo += size
+
+
+def _runs_of(kv_offs, kv_lens, q_offs, q_lens, q_entries):
+    """The (KV run, request list) pairs behind the planner's vnodes.
+
+    Vnodes over one KV slice whose scratch rows adjoin are the query tiles of one chunk
+    (kernel_bench/fasttree.py:212-231); chunks whose slices adjoin and whose requests are equal
+    are the KV splits of one node (fasttree.py:199-210).  Returns a list of
+    ``(kv_start, chunk_lens, requests)``: the run starts at ``kv_start`` of the flat KV index
+    list and was cut by the planner into chunks of ``chunk_lens`` tokens.
+    """
+    n = len(kv_offs)
+    order = np.lexsort((q_offs, kv_lens, kv_offs))
+    chunks = []   # (kv_off, kv_len, requests)
+    i = 0
+    while i < n:
+        v = order[i]
+        reqs = [q_entries[q_offs[v]: q_offs[v] + q_lens[v]]]
+        end = q_offs[v] + q_lens[v]
+        j = i + 1
+        while j < n:
+            w = order[j]
+            if kv_offs[w] != kv_offs[v] or kv_lens[w] != kv_lens[v] or q_offs[w] != end:
+                break
+            reqs.append(q_entries[q_offs[w]: q_offs[w] + q_lens[w]])
+            end = q_offs[w] + q_lens[w]
+            j += 1
+        chunks.append((int(kv_offs[v]), int(kv_lens[v]), np.concatenate(reqs)))
+        i = j
+    # chain the chunks of one node: the next chunk starts where this one ends, same requests
+    by_start = {}
+    for idx, (off, length, reqs) in enumerate(chunks):
+        by_start.setdefault(off, []).append(idx)
+    follower = [-1] * len(chunks)
+    has_leader = [False] * len(chunks)
+    for idx, (off, length, reqs) in enumerate(chunks):
+        if length == 0:
+            continue
+        for cand in by_start.get(off + length, ()):
+            if cand != idx and not has_leader[cand] and np.array_equal(chunks[cand][2], reqs):
+                follower[idx] = cand
+                has_leader[cand] = True
+                break
+    runs = []
+    for idx in range(len(chunks)):
+        if has_leader[idx]:
+            continue
+        lens, cur = [], idx
+        while cur >= 0:
+            lens.append(chunks[cur][1])
+            cur = follower[cur]
+        runs.append((chunks[idx][0], lens, chunks[idx][2]))
+    return runs
+
+
+def block_programs(kv_offs, kv_lens, q_offs, q_lens, q_entries, batch_size, group, num_kv_heads, *,
+                   block_rows=BLOCK_ROWS, block_slots=None, recut=None, embed=False, head_dim=128) -> LaunchSchedule:
+    """The planner's lists arranged as equal-work block programs (see the module docstring).
+
+    With ``block_slots=None`` the launch is laid out twice, for programs on every block slot of
+    the machine (two per compute unit: the narrow vnodes then wait for the programs to end) and
+    on half of them (one per compute unit: the narrow vnodes run beside the programs from the
+    start, and a program that has its compute unit to itself steps faster), and the layout with
+    the shorter modelled duration is returned.
+    """
+    if block_slots is None:
+        both = [_block_programs(kv_offs, kv_lens, q_offs, q_lens, q_entries, batch_size, group, num_kv_heads,
+                                block_rows=block_rows, block_slots=slots, recut=recut, embed=embed, head_dim=head_dim)
+                for slots in (BLOCK_SLOTS, BLOCK_SLOTS // 2)]
+        return min(both, key=lambda sched: sched.modelled_us)
+    return _block_programs(kv_offs, kv_lens, q_offs, q_lens, q_entries, batch_size, group, num_kv_heads,
+                           block_rows=block_rows, block_slots=block_slots, recut=recut, embed=embed, head_dim=head_dim)
+
+
+def _block_programs(kv_offs, kv_lens, q_offs, q_lens, q_entries, batch_size, group, num_kv_heads, *,
+                    block_rows, block_slots, recut, embed, head_dim) -> LaunchSchedule:
+    """One layout of :func:`block_programs`, for ``block_slots`` programs at a time.
+
+    Takes the four per-vnode lists and the scratch-row list of kernel_bench/fasttree.py:193-231
+    (any order), the number of requests, the GQA group size and the number of KV heads.
+    ``recut`` forces (True) or forbids (False) cutting the wide runs anew; by default they are
+    cut anew when every program of one round gets at least :data:`MIN_PROGRAM_TILES` of work.
+    ``embed`` deals the narrow vnodes to the programs (None: when the runs were cut anew and no
+    program's share outweighs its wide vnodes).  Off by default: measured, a program block that
+    has its compute unit to itself steps only about a fifth faster, so narrow vnodes inside the
+    programs run one after the other with the wide work all the same.
+    """
+    kv_offs, kv_lens, q_offs, q_lens = (np.asarray(x, dtype=np.int64) for x in (kv_offs, kv_lens, q_offs, q_lens))
+    q_entries = np.asarray(q_entries, dtype=np.int64)
+    group = max(1, int(group))
+    heads = max(1, int(num_kv_heads))
+    cap = max(1, int(block_rows) // group)            # requests per row chunk
+    per_round = max(1, int(block_slots) // heads)     # programs per round and head
+
+    runs = _runs_of(kv_offs, kv_lens, q_offs, q_lens, q_entries)
+    wide_runs, narrow = [], []    # narrow: (kv_off, kv_len, requests) per planner chunk
+    for start, lens, reqs in runs:
+        rows = len(reqs) * group
+        if rows <= NARROW_ROWS:
+            off = start
+            for length in lens:
+                narrow.append((off, length, reqs))
+                off += length
+        else:
+            wide_runs.append((start, lens, reqs))
+    # light wide runs go with the narrow vnodes when the wide blocks alone overfill the machine
+    wide_blocks = sum(len(lens) * -(-len(reqs) * group // block_rows) for _, lens, reqs in wide_runs) * heads
+    if wide_blocks > block_slots:
+        kept = []
+        for start, lens, reqs in wide_runs:
+            rows = len(reqs) * group
+            if rows <= LIGHT_ROWS and rows * max(lens) <= LIGHT_WORK:
+                off = start
+                for length in lens:
+                    narrow.append((off, length, reqs))
+                    off += length
+            else:
+                kept.append((start, lens, reqs))
+        wide_runs = kept
+
+    # ---- work items: (run, row chunk) with the run's planner chunks as possible cut points
+    def tiles(tokens):
+        return -(-tokens // TILE_TOKENS)
+
+    items = []   # (weight per tile, kv_start, chunk_lens, requests of the row chunk)
+    for start, lens, reqs in wide_runs:
+        for lo, hi in _row_chunks(len(reqs), cap):
+            part = reqs[lo:hi]
+            items.append((_tile_weight(len(part) * group), start, lens, part))
+    total = sum(w * tiles(sum(lens)) + VNODE_STARTUP_TILES for w, _, lens, _ in items)
+    do_recut = (total / per_round >= MIN_PROGRAM_TILES) if recut is None else bool(recut)
+
+    pieces = []      # (kv_off, kv_len, requests, work)
+    programs = []    # list of lists of piece indices
+    if items and do_recut:
+        rounds = max(1, int(np.ceil(total / (per_round * MAX_PROGRAM_TILES))))
+        nprog = per_round * rounds
+        items.sort(key=lambda it: -(it[0] * tiles(sum(it[2]))))
+
+        def fill(target):
+            """Programs filled to `target` one after the other, runs cut where a program is full."""
+            pieces, programs, current, load = [], [], [], 0.0
+            for w, start, lens, part in items:
+                run_len, done = sum(lens), 0
+                while done < run_len:
+                    left = run_len - done
+                    last = len(programs) >= nprog - 1          # the last program takes whatever is left
+                    room = target - load - VNODE_STARTUP_TILES  # tile steps of this weight that still fit
+                    fit = (int(room / w) * TILE_TOKENS) // CUT_TOKENS * CUT_TOKENS if room > 0 else 0
+                    if last or fit >= left or left - fit < MIN_PIECE_TOKENS:
+                        take = left                              # the rest fits (or what would remain is too short)
+                    elif fit >= MIN_PIECE_TOKENS:
+                        take = fit                               # the program is full here
+                    elif current:
+                        programs.append((current, load))         # no room worth a piece: next program
+                        current, load = [], 0.0
+                        continue
+                    else:
+                        take = left
+                    work = w * tiles(take) + VNODE_STARTUP_TILES
+                    current.append(len(pieces))
+                    pieces.append((start + done, take, part, work))
+                    load += work
+                    done += take
+                    if load >= target - 0.5 * w and not last:
+                        programs.append((current, load))
+                        current, load = [], 0.0
+            if current:
+                programs.append((current, load))
+            return pieces, programs
+
+        # the smallest target (within a few percent) that the last program does not overshoot:
+        # every cut adds a vnode and its start-up charge, so the first guess is a lower bound
+        target = total / nprog
+        for _ in range(60):
+            pieces, filled = fill(target)
+            if max(load for _, load in filled) <= 1.04 * target:
+                break
+            target *= 1.03
+        programs = [prog for prog, _ in filled]
+    elif items:
+        # The planner's chunks as they are, one vnode per program, longest first.  While the
+        # launch would leave half of the machine idle, row chunks are halved (down to 64 rows):
+        # the block's waves then split the tokens of the smaller chunk among them.
+        rows_cap = int(block_rows)
+        while rows_cap > 64:
+            cap_now = max(1, rows_cap // group)
+            blocks = sum(len(lens) * -(-len(reqs) // cap_now) for _, lens, reqs in wide_runs) * heads
+            if 2 * blocks > block_slots:
+                break
+            rows_cap //= 2
+        cap_now = max(1, rows_cap // group)
+        for start, lens, reqs in wide_runs:
+            for lo, hi in _row_chunks(len(reqs), cap_now):
+                part = reqs[lo:hi]
+                w = _tile_weight(len(part) * group)
+                off = start
+                for length in lens:
+                    pieces.append((off, length, part, w * tiles(length) + VNODE_STARTUP_TILES))
+                    off += length
+        order = sorted(range(len(pieces)), key=lambda i: -pieces[i][3])
+        programs = [[i] for i in order]
+
+    # ---- narrow vnodes, longest first; dealt to the programs when those fill the machine
+    def narrow_work(v):
+        return NARROW_STARTUP_TILES + NARROW_STEP_TILES * tiles(v[1]) * -(-len(v[2]) * group // NARROW_ROWS)
+
+    narrow.sort(key=lambda v: -narrow_work(v))
+    program_tiles = [sum(pieces[i][3] for i in prog) for prog in programs]
+    shares = [[] for _ in programs]
+    embed_narrow = embed if embed is not None else (do_recut and bool(programs) and bool(narrow))
+    if embed_narrow and programs and narrow:
+        nprog = len(programs)
+        for i, v in enumerate(narrow):
+            lap, pos = divmod(i, nprog)
+            shares[pos if lap % 2 == 0 else nprog - 1 - pos].append(v)
+        # a program's waves serve its share together: the share takes as long as its largest wave load
+        waves = BLOCK_WAVES
+        share_tiles = [max(sum(narrow_work(v) for v in sh[w::waves]) for w in range(waves)) if sh else 0.0
+                       for sh in shares]
+        if embed is None and max(share_tiles) > min(program_tiles):
+            shares = [[] for _ in programs]     # the narrow vnodes outweigh the programs: blocks of their own
+        else:
+            program_tiles = [t + s for t, s in zip(program_tiles, share_tiles)]
+    embedded = [v for sh in shares for v in sh]
+    taken = {id(v) for v in embedded}
+    narrow = embedded + [v for v in narrow if id(v) not in taken]
+
+    # ---- the lists: wide pieces in program order, then the narrow vnodes
+    new_kv_offs, new_kv_lens, new_q_offs, new_q_lens, rows_out = [], [], [], [], []
+    prog_table = []
+    row = 0
+
+    def emit(off, length, reqs):
+        nonlocal row
+        new_kv_offs.append(off)
+        new_kv_lens.append(length)
+        new_q_offs.append(row)
+        new_q_lens.append(len(reqs))
+        rows_out.append(reqs)
+        row += len(reqs)
+
+    narrow_first = 0
+    for p, prog in enumerate(programs):
+        wide_first = len(new_kv_offs)
+        for i in prog:
+            emit(*pieces[i][:3])
+        # the two blocks of a compute unit (block b and b + 256) get opposite orders
+        front = (p % per_round) < per_round // 2
+        prog_table.append((wide_first, len(new_kv_offs), narrow_first, -len(shares[p]) if front else len(shares[p])))
+        narrow_first += len(shares[p])
+    n_wide = len(new_kv_offs)
+    for off, length, reqs in narrow:
+        emit(off, length, reqs)
+    new_q_entries = np.concatenate(rows_out) if rows_out else np.zeros(0, dtype=np.int64)
+
+    # scratch rows of every request, in row order (kernel_bench/fasttree.py:233-244)
+    by_req = np.argsort(new_q_entries, kind="stable")
+    req_lens = np.bincount(new_q_entries, minlength=int(batch_size)).astype(np.int64)[: int(batch_size)]
+    req_offs = np.concatenate([[0], np.cumsum(req_lens)[:-1]]) if batch_size else np.zeros(0, dtype=np.int64)
+    req_entries = np.concatenate([by_req, np.full(32, -1, dtype=np.int64)])
+
+    # ---- modelled duration of the launch (microseconds)
+    shared = len(programs) * heads > BLOCK_SLOTS // 2          # two program blocks on some compute unit
+    tile_us = TILE_US_SHARED if shared else TILE_US_ALONE
+    if programs:
+        waves_of_blocks = max(1.0, len(programs) * heads / float(block_slots))
+        wide_us = max(max(program_tiles), sum(program_tiles) / len(programs) * waves_of_blocks) * tile_us
+    else:
+        wide_us = 0.0
+    trailing = narrow[narrow_first:]
+    if trailing:
+        item_us = [narrow_work(v) * TILE_US_SHARED for v in trailing]
+        narrow_bytes = sum(v[1] for v in trailing) * heads * 4 * head_dim
+        slots_for_narrow = WAVE_SLOTS if shared or not programs else WAVE_SLOTS // 2
+
+        def narrow_us(wave_slots):
+            return max(sum(item_us) * heads / wave_slots, max(item_us), narrow_bytes / NARROW_BYTES_PER_US)
+
+        modelled = wide_us + narrow_us(WAVE_SLOTS) if shared else max(wide_us, narrow_us(slots_for_narrow))
+    else:
+        modelled = wide_us
+
+    i32 = lambda x: np.asarray(x, dtype=np.int32)
+    return LaunchSchedule(
+        kv_offs=i32(new_kv_offs), kv_lens=i32(new_kv_lens), q_offs=i32(new_q_offs), q_lens=i32(new_q_lens),
+        q_entries=i32(new_q_entries), req_entries=i32(req_entries), req_offs=i32(req_offs), req_lens=i32(req_lens),
+        phase_node_nums=[n_wide, len(new_kv_offs) - n_wide], phase_node_offsets=[0, n_wide],
+        prog_table=i32(prog_table).reshape(-1, 4), narrow_in_programs=narrow_first,
+        program_tiles=np.asarray(program_tiles, dtype=np.float64), block_slots=int(block_slots),
+        modelled_us=float(modelled),
+    )

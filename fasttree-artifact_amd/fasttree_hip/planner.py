@@ -421,279 +421,6 @@ def fasttree_plan(
     )
 
 
-#: A first-phase vnode of at most LIGHT_VNODE_ROWS query rows and LIGHT_VNODE_WORK query rows x
-#: KV tokens is launched with the second phase when the first phase alone has more blocks than
-#: WIDE_BLOCK_SLOTS, the number an MI355X runs at a time (256 compute units x 2); see
-#: :func:`vnodes_in_launch_order`.
-LIGHT_VNODE_WORK = 4096
-LIGHT_VNODE_ROWS = 64
-WIDE_BLOCK_SLOTS = 512
-
-
-#: Query rows one block of the first-phase kernel serves per pass.
-WIDE_BLOCK_ROWS = 128
-
-
-def vnodes_in_launch_order(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, phase_node_offsets, group,
-                           num_kv_heads=None, light_work=None, q_tile=None, return_order=False):
-    """The four per-vnode lists and the two phase lists, rearranged for the decode kernels.
-
-    A vnode is the tuple (kv_offs[v], kv_lens[v], q_offs[v], q_lens[v]); nothing else refers to
-    a vnode by its position (the per-request lists of kernel_bench/fasttree.py:233-244 name
-    scratch rows, not vnodes), and the kernels compute a vnode of any number of query rows in
-    either phase, so the order within a phase and the phase a vnode is launched with change the
-    schedule, not the result.  Three changes against the reference's order (fasttree.py:246-259):
-
-    * light first-phase vnodes -- at most :data:`LIGHT_VNODE_ROWS` query rows and query rows x
-      KV tokens at most ``light_work`` (default :data:`LIGHT_VNODE_WORK`) -- move to the second
-      phase, provided the first phase has more blocks (vnodes x ``num_kv_heads``) than the
-      machine runs at a time (:data:`WIDE_BLOCK_SLOTS`; always, when ``num_kv_heads`` is None).
-      A first-phase vnode gets a block of four waves with a staging ring for long runs, two
-      blocks per compute unit; a second-phase vnode gets one wave that serves 16 rows per
-      pass, eight or more per compute unit.  Short runs under a few dozen rows are bound by
-      memory latency, not by arithmetic: when there are more of them than block slots, they
-      finish sooner with more of them in flight; when there are fewer, a block's four waves
-      finish one sooner than a single wave's passes do.
-    * the second phase is listed in order of decreasing work (KV tokens x passes of 16 rows;
-      equal work keeps the order).  The kernel hands these vnodes to the machine in list order,
-      each to one wave that walks its run tile by tile: a long run that starts last is what the
-      launch then waits for.
-    * with ``q_tile`` (the first phase's query tile, in requests) given: neighbours in the
-      first phase that attend the same KV run with adjoining scratch rows -- the query tiles one
-      node was cut into (fasttree.py:212-231) -- are joined into one vnode of at most
-      ``WIDE_BLOCK_ROWS x ceil(q_tile x group / WIDE_BLOCK_ROWS)`` query rows, what the blocks of
-      one vnode serve in a single pass: a tile of 16 requests x 4 heads fills half of a block's
-      rows, and two such tiles would stage the same run twice.  Not done while the first phase
-      has no more blocks than the machine has compute units (two half-filled blocks side by
-      side finish sooner than one full block).  The kernel joins such neighbours itself when
-      it is handed the reference's lists; joined here, no block is launched for the tiles
-      that were absorbed.
-
-    The order within the first phase is otherwise left alone (the kernel ranks those vnodes
-    itself).  Returns ``(kv_offs, kv_lens, q_offs, q_lens, phase_node_nums, phase_node_offsets)``;
-    with ``return_order`` a seventh element: for every vnode of the input its position in the
-    output, or -1 for a query tile that was absorbed into its neighbour.
-    """
-    light_work = LIGHT_VNODE_WORK if light_work is None else light_work
-    lists = [np.array(x, dtype=np.int32, copy=True) for x in (kv_offs, kv_lens, q_offs, q_lens)]
-    first, count0, count1 = int(phase_node_offsets[0]), int(phase_node_nums[0]), int(phase_node_nums[1])
-    if first != 0 or int(phase_node_offsets[1]) != count0:
-        raise ValueError("the phases must be adjoining ranges starting at vnode 0")
-    rows = lists[3].astype(np.int64) * int(group)
-    tokens = lists[1].astype(np.int64)
-    index = np.arange(count0 + count1)
-    light = (index < count0) & (rows * tokens <= light_work) & (rows <= LIGHT_VNODE_ROWS)
-    if num_kv_heads is not None and count0 * int(num_kv_heads) <= WIDE_BLOCK_SLOTS:
-        light[:] = False
-    wide = index[(index < count0) & ~light]
-    narrow = np.concatenate([index[light], index[count0:]])
-    work = tokens[narrow] * ((rows[narrow] + 15) // 16)
-    narrow = narrow[np.argsort(-work, kind="stable")]
-    order = np.concatenate([wide, narrow])
-    lists = [x[order] for x in lists]
-    n_wide = len(wide)
-    kept_all = np.arange(len(order))
-    if q_tile is not None and n_wide > 1:
-        chunks = max(1, min(8, (int(q_tile) * int(group) + WIDE_BLOCK_ROWS - 1) // WIDE_BLOCK_ROWS))
-        heads = 1 if num_kv_heads is None else int(num_kv_heads)
-        if num_kv_heads is None or 2 * n_wide * heads * chunks > WIDE_BLOCK_SLOTS:
-            cap = WIDE_BLOCK_ROWS * chunks // int(group)  # requests
-            kept = [0]
-            kv_o, kv_l, q_o, q_l = (x[:n_wide].astype(np.int64) for x in lists)
-            q_l = q_l.copy()
-            for v in range(1, n_wide):
-                h = kept[-1]
-                if (kv_o[v] == kv_o[h] and kv_l[v] == kv_l[h] and q_o[h] + q_l[h] == q_o[v]
-                        and q_l[h] + q_l[v] <= cap):
-                    q_l[h] += q_l[v]
-                else:
-                    kept.append(v)
-            lists[3][:n_wide] = q_l.astype(np.int32)
-            keep = np.concatenate([np.array(kept, dtype=np.int64), np.arange(n_wide, len(order))])
-            lists = [x[keep] for x in lists]
-            n_wide = len(kept)
-            kept_all = keep
-    result = (*lists, [n_wide, len(narrow)], [0, n_wide])
-    if return_order:
-        where = np.full(len(order), -1, dtype=np.int64)
-        where[order[kept_all]] = np.arange(len(kept_all))
-        result = (*result, where)
-    return result
-
-
-#: Blocks (128-row blocks x kv heads) the vnodes of one KV run must make for the run's KV split to
-#: be undone: one per compute unit of an MI355X; see :func:`join_kv_chunks`.
-FULL_MACHINE_BLOCKS = 256
-
-#: First-phase blocks a launch may have for all of them to be resident at once with a few block
-#: slots to spare (of :data:`WIDE_BLOCK_SLOTS`); see :func:`join_kv_chunks`.
-RESIDENT_WIDE_BLOCKS = 472
-
-
-def join_kv_chunks(kv_offs, kv_lens, q_offs, q_lens, q_entries, req_entries, req_offs, req_lens,
-                   phase_node_nums, phase_node_offsets, group, num_kv_heads, min_blocks=None, resident_blocks=None,
-                   return_order=False):
-    """Cuts long KV runs into fewer chunks than the planner did where the chunks buy nothing.
-
-    The planner cuts every run into chunks of the phase's KV split size whatever the number of
-    requests under it (kernel_bench/fasttree.py:199-231): chunk s of a node is served by its own
-    vnodes over its own copy of the node's scratch rows, and the second stage merges the copies
-    per request.  The split buys parallelism, and each chunk costs a partial row per request and
-    head to write, read and merge.  Two cases where fewer chunks are better:
-
-    * a run attended by so many query rows that the 128-row blocks x kv heads of ONE chunk
-      already number ``min_blocks`` (default :data:`FULL_MACHINE_BLOCKS`) has its parallelism
-      without the split: it becomes one chunk;
-    * a launch whose first phase has a few more blocks than the machine holds at once
-      (``resident_blocks``, default :data:`RESIDENT_WIDE_BLOCKS`) runs its last blocks behind the
-      others and keeps the second phase's short vnodes waiting for a block slot; when longer
-      chunks bring the first phase under that number, the chunked runs are cut at the shortest
-      common chunk length that does (C3: three chunks of its 4000-token root instead of four,
-      472 blocks instead of 576).  Only runs whose blocks still number nine tenths of
-      ``min_blocks`` afterwards are cut anew: a few long blocks on an otherwise idle machine
-      would cost more.
-
-    Where a vnode's KV slice ends the next chunk's begins (the flat KV index list holds a node's
-    tokens back to back); vnodes over that next slice that serve the same requests in the same
-    tiles are the next chunk.  A chain of S chunks that is to have S' < S is cut anew into S'
-    equal slices (multiples of 64 tokens) served by the vnodes of its first S' chunks; the vnodes
-    of the others are dropped together with their scratch rows, which leave the per-request
-    lists (the rows stay allocated and unused).
-
-    Takes the lists in the planner's order (first phase, then second) and returns
-    ``(kv_offs, kv_lens, q_offs, q_lens, req_entries, req_offs, req_lens, phase_node_nums,
-    phase_node_offsets)`` with ``req_entries`` padded by 32 x -1 as the planner's
-    (fasttree.py:261-262); the inputs are not modified.  With ``return_order`` a tenth
-    element: for every vnode of the input its position in the output, or -1 if it was dropped.
-    """
-    min_blocks = FULL_MACHINE_BLOCKS if min_blocks is None else int(min_blocks)
-    resident = RESIDENT_WIDE_BLOCKS if resident_blocks is None else int(resident_blocks)
-    kv_o, kv_l, q_o, q_l = (np.array(x, dtype=np.int64, copy=True) for x in (kv_offs, kv_lens, q_offs, q_lens))
-    heads = max(1, int(num_kv_heads))
-    count0 = int(phase_node_nums[0])
-    n = len(kv_o)
-
-    def unchanged():
-        out = (kv_o.astype(np.int32), kv_l.astype(np.int32), q_o.astype(np.int32), q_l.astype(np.int32),
-               np.asarray(req_entries, dtype=np.int32), np.asarray(req_offs, dtype=np.int32),
-               np.asarray(req_lens, dtype=np.int32), list(phase_node_nums), list(phase_node_offsets))
-        return (*out, np.arange(n, dtype=np.int64)) if return_order else out
-
-    if n == 0:
-        return unchanged()
-    # blocks per run (the vnodes over one KV slice): requests summed over its vnodes
-    _, first_of, run_of = np.unique((kv_o << 32) | kv_l, return_index=True, return_inverse=True)
-    run_rows = np.bincount(run_of, weights=q_l).astype(np.int64) * int(group)
-    run_blocks = -(-run_rows // WIDE_BLOCK_ROWS) * heads
-    wide_total = int(run_blocks[first_of < count0].sum())  # (a run's vnodes share a phase but for a narrow last tile)
-    full = run_blocks >= min_blocks
-    if not full.any() and wide_total <= resident:
-        return unchanged()
-    # candidates: runs that another run follows or that follow another run
-    run_start, run_end = kv_o[first_of], kv_o[first_of] + kv_l[first_of]
-    chained = np.isin(run_end, run_start) | np.isin(run_start, run_end)
-    if not chained.any():
-        return unchanged()
-    q_ent = np.asarray(q_entries, dtype=np.int64)
-    runs = {}
-    for v in np.nonzero(chained[run_of])[0].tolist():
-        runs.setdefault((int(kv_o[v]), int(kv_l[v])), []).append(v)
-    starts = {}
-    for key in runs:
-        starts.setdefault(key[0], []).append(key)
-    chains, taken = [], set()
-    for key in sorted(runs):
-        if key in taken:
-            continue
-        chain, tiles, end = [key], runs[key], key[0] + key[1]
-        while True:
-            follower = None
-            for cand in starts.get(end, ()):
-                other = runs[cand]
-                if cand in taken or cand == key or len(other) != len(tiles):
-                    continue
-                if all(q_l[a] == q_l[b] and (a < count0) == (b < count0)
-                       and np.array_equal(q_ent[q_o[a]: q_o[a] + q_l[a]], q_ent[q_o[b]: q_o[b] + q_l[b]])
-                       for a, b in zip(tiles, other)):
-                    follower = cand
-                    break
-            if follower is None:
-                break
-            taken.add(follower)
-            chain.append(follower)
-            end = follower[0] + follower[1]
-        if len(chain) > 1:
-            rows = int(q_l[tiles].sum()) * int(group)
-            chains.append((-(-rows // WIDE_BLOCK_ROWS) * heads, chain))
-    # how many chunks each chain keeps
-    plan = []
-    for per, chain in chains:
-        if per >= min_blocks:
-            plan.append((per, chain, 1))
-            if runs[chain[0]][0] < count0:
-                wide_total -= per * (len(chain) - 1)
-    if wide_total > resident:
-        # One chunk length for all: the shortest for which the phase fits, every run that is cut
-        # anew still covering the machine by itself (its blocks number nine tenths of min_blocks
-        # or more; runs that cannot are left as they are -- a few long blocks on an otherwise
-        # idle machine would be what the launch waits for).
-        covering = max(1, 9 * min_blocks // 10)
-        rest = []
-        for per, chain in chains:
-            fewest = -(-covering // per)
-            if per < min_blocks and runs[chain[0]][0] < count0 and fewest < len(chain):
-                rest.append((per, chain, sum(key[1] for key in chain), fewest))
-        fixed = wide_total - sum(per * len(chain) for per, chain, _, _ in rest)
-
-        def chunks_at(length):
-            return [min(len(chain), max(fewest, -(-tokens // length))) for _, chain, tokens, fewest in rest]
-
-        lengths = sorted({-(-tokens // k) for _, chain, tokens, fewest in rest for k in range(fewest, len(chain) + 1)})
-        for length in lengths:
-            keeps = chunks_at(length)
-            if fixed + sum(per * keep for (per, _, _, _), keep in zip(rest, keeps)) <= resident:
-                plan += [(per, chain, keep) for (per, chain, _, _), keep in zip(rest, keeps) if keep < len(chain)]
-                break
-    dropped = np.zeros(n, dtype=bool)
-    for per, chain, keep in plan:
-        start = chain[0][0]
-        total = sum(key[1] for key in chain)
-        size = -(-(-(-total // keep)) // 64) * 64  # ceil(total / keep), up to a multiple of 64
-        for i, key in enumerate(chain):
-            if i < keep and i * size < total:
-                kv_o[runs[key]] = start + i * size
-                kv_l[runs[key]] = min(size, total - i * size)
-            else:
-                dropped[runs[key]] = True
-    if not dropped.any():
-        return unchanged()
-    entries = np.asarray(req_entries, dtype=np.int64)
-    lens = np.asarray(req_lens, dtype=np.int64)
-    offs = np.asarray(req_offs, dtype=np.int64)
-    total = int(lens.sum())
-    if not np.array_equal(offs, np.concatenate([[0], np.cumsum(lens)[:-1]])):
-        raise ValueError("the per-request lists must lie back to back in request order")
-    row_dropped = np.zeros(len(q_ent), dtype=bool)
-    for v in np.nonzero(dropped)[0]:
-        row_dropped[q_o[v]: q_o[v] + q_l[v]] = True
-    listed = entries[:total]
-    keep = ~row_dropped[listed]
-    owner = np.repeat(np.arange(len(lens)), lens)
-    new_lens = np.bincount(owner[keep], minlength=len(lens))
-    new_offs = np.concatenate([[0], np.cumsum(new_lens)[:-1]])
-    new_entries = np.concatenate([listed[keep], np.full(32, -1, dtype=np.int64)])
-    kept = ~dropped
-    n0 = int(kept[:count0].sum())
-    out = (kv_o[kept].astype(np.int32), kv_l[kept].astype(np.int32), q_o[kept].astype(np.int32), q_l[kept].astype(np.int32),
-           new_entries.astype(np.int32), new_offs.astype(np.int32), new_lens.astype(np.int32),
-           [n0, int(kept.sum()) - n0], [0, n0])
-    if return_order:
-        where = np.full(n, -1, dtype=np.int64)
-        where[kept] = np.arange(int(kept.sum()))
-        out = (*out, where)
-    return out
-
-
 class PlanBuffers:
     """Device buffers for :func:`fasttree_preparation`, allocated once at stated maxima and
     filled in place by every call that is given them: a serving loop re-plans whenever its batch
@@ -719,6 +446,7 @@ class PlanBuffers:
         self.vnode_to_q_offs, self.vnode_to_q_lens = ints(max_vnodes), ints(max_vnodes)
         self.req_to_vnode_entries = ints(max_rows + 32)
         self.req_to_vnode_offs, self.req_to_vnode_lens = ints(max_batch_size), ints(max_batch_size)
+        self.prog_table = ints(4 * max_vnodes)
         self.mid_o = torch.empty((int(max_rows), num_qo_heads, head_dim), dtype=torch.float32, device=device)
         self.mid_lse = torch.empty((int(max_rows), num_qo_heads), dtype=torch.float32, device=device)
 
@@ -749,7 +477,7 @@ def fasttree_preparation(
     *,
     device="cuda",
     kv_slot_map=None,
-    launch_order=True,
+    launch_order=False,
     buffers=None,
 ):
     """Drop-in for kernel_bench/fasttree.py:99-296: plan on the host, then place the nine
@@ -758,14 +486,20 @@ def fasttree_preparation(
     Returns ``((vnode_to_kv_entries, vnode_to_kv_offs, vnode_to_kv_lens,
     vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, req_to_vnode_entries,
     req_to_vnode_offs, req_to_vnode_lens, mid_o, mid_lse, phase_node_nums,
-    phase_node_offsets), node_assignments)``.  The keyword-only arguments do not exist
-    in the reference: ``device`` defaults to the reference's hard-wired "cuda";
-    ``kv_slot_map`` is described in :func:`fasttree_plan`; ``launch_order`` arranges the vnodes
-    for the kernels (:func:`join_kv_chunks`, then :func:`vnodes_in_launch_order`) instead of
-    leaving them in the reference's order; with ``buffers`` (a :class:`PlanBuffers`) nothing is allocated on the device: the
-    arrays are written into its buffers and the returned tensors are their leading parts.
+    phase_node_offsets), node_assignments)``: element for element the reference's lists.
+
+    The keyword-only arguments do not exist in the reference: ``device`` defaults to the
+    reference's hard-wired "cuda"; ``kv_slot_map`` is described in :func:`fasttree_plan`; with
+    ``buffers`` (a :class:`PlanBuffers`) nothing is allocated on the device: the arrays are
+    written into its buffers and the returned tensors are their leading parts.  With
+    ``launch_order=True`` the lists come back arranged for an MI355X instead
+    (:func:`launch_schedule.block_programs`: the same computation as equal-work block programs,
+    with scratch rows and per-request lists of its own); ``phase_node_nums`` is then a list that
+    also carries the program table, which ``fasttree_decode`` picks up.
     """
     import torch
+
+    from .launch_schedule import LaunchPhases, block_programs
 
     plan = fasttree_plan(
         tree_info, KV_ptrs, batch_size, num_kv_heads,
@@ -775,22 +509,32 @@ def fasttree_preparation(
     names = iter(("vnode_to_kv_entries", "vnode_to_kv_offs", "vnode_to_kv_lens", "vnode_to_q_entries", "vnode_to_q_offs",
                   "vnode_to_q_lens", "req_to_vnode_entries", "req_to_vnode_offs", "req_to_vnode_lens"))
 
-    def put(values):
-        name = next(names)  # (the nine arrays are placed in this order below)
+    def place(name, values):
         if buffers is not None:
             return buffers.fill(name, values)
         host = torch.from_numpy(np.ascontiguousarray(np.asarray(values, dtype=np.int32)))
         return host.to(device)
 
+    def put(values):
+        return place(next(names), values)  # (the nine arrays are placed in this order below)
+
     rows = plan.num_rows
-    vnodes = (plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens,
-              plan.phase_node_nums, plan.phase_node_offsets)
+    vnodes = (plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens)
+    q_entries = plan.vnode_to_q_entries
     per_request = (plan.req_to_vnode_entries, plan.req_to_vnode_offs, plan.req_to_vnode_lens)
+    phase_nums, phase_offs = list(plan.phase_node_nums), list(plan.phase_node_offsets)
     if launch_order:
         group = max(1, num_qo_heads // num_kv_heads)
-        joined = join_kv_chunks(*vnodes[:4], plan.vnode_to_q_entries, *per_request, *vnodes[4:], group, num_kv_heads)
-        vnodes, per_request = (*joined[:4], *joined[7:]), joined[4:7]
-        vnodes = vnodes_in_launch_order(*vnodes, group, num_kv_heads, q_tile=params.TSQs[0])
+        sched = block_programs(*vnodes, q_entries, batch_size, group, num_kv_heads)
+        vnodes = (sched.kv_offs, sched.kv_lens, sched.q_offs, sched.q_lens)
+        q_entries = sched.q_entries
+        per_request = (sched.req_entries, sched.req_offs, sched.req_lens)
+        rows = sched.num_rows
+        phase_nums, phase_offs = LaunchPhases(sched.phase_node_nums), list(sched.phase_node_offsets)
+        if sched.num_programs > 0:
+            phase_nums.prog_table = place("prog_table", sched.prog_table.reshape(-1))
+            phase_nums.num_programs = sched.num_programs
+            phase_nums.narrow_in_programs = sched.narrow_in_programs
     if buffers is not None:
         if rows > buffers.mid_o.shape[0] or buffers.mid_o.shape[1:] != (num_qo_heads, head_dim):
             raise ValueError(f"the scratch of the buffers ({tuple(buffers.mid_o.shape)}) does not hold "
@@ -803,7 +547,7 @@ def fasttree_preparation(
         put(plan.vnode_to_kv_entries),
         put(vnodes[0]),
         put(vnodes[1]),
-        put(plan.vnode_to_q_entries),
+        put(q_entries),
         put(vnodes[2]),
         put(vnodes[3]),
         put(per_request[0]),
@@ -811,7 +555,7 @@ def fasttree_preparation(
         put(per_request[2]),
         mid_o,
         mid_lse,
-        list(vnodes[4]),
-        list(vnodes[5]),
+        phase_nums,
+        phase_offs,
     )
     return aux, plan.node_assignments

@@ -68,8 +68,8 @@ class FastTreeMetadata:
         #: not in the reference: the hook writes the step's K/V rows with this library's single
         #: launch instead of calling the layer's ``store_kv_cache``
         self.fused_store = fused_store
-        #: not in the reference: the vnode lists are arranged for the kernels
-        #: (planner.vnodes_in_launch_order) instead of left in the reference's order
+        #: not in the reference: the vnode lists are arranged as block programs for the kernels
+        #: (launch_schedule.block_programs) instead of left in the reference's order
         self.launch_order = launch_order
 
         def ints(n):
@@ -85,6 +85,8 @@ class FastTreeMetadata:
         self.req_to_vnode_lens = ints(max_batch_size)
         self.mid_o = torch.empty((max_vnode_to_q_entries, num_qo_heads, head_dim), dtype=torch.float32, device=device)
         self.mid_lse = torch.empty((max_vnode_to_q_entries, num_qo_heads), dtype=torch.float32, device=device)
+        #: not in the reference: the block programs of a launch-order plan (four entries each)
+        self.prog_table = ints(4 * max_vnodes)
 
         self.phase_node_nums: Optional[Sequence[int]] = None
         self.phase_node_offsets: Optional[Sequence[int]] = None
@@ -273,30 +275,38 @@ def prepare_for_fasttree_meta(batch, fasttree_metadata: FastTreeMetadata):
     meta.phase_node_nums = [len(above), len(below)]
     meta.phase_node_offsets = [0, len(above)]
     lists = [[x[i] for i in perm] for x in (kv_offs, kv_lens, q_offs, q_lens)]
+    meta.prog_table_len = 0
     if getattr(meta, "launch_order", False):
-        from .planner import join_kv_chunks, vnodes_in_launch_order
+        from .launch_schedule import LaunchPhases, block_programs
 
-        # long shared runs in fewer KV chunks where the chunks buy nothing (a system prompt under
-        # a large batch), then the vnodes in launch order
+        # the same computation as equal-work block programs: long shared runs (a system prompt
+        # under a large batch) cut where the machine is full instead of at the KV split
         tail_ends = [lists[0][v] + lists[1][v] for v in meta.req_last_vnodes]
-        *lists, req_entries, req_offs, req_lens, nums, offs, kept = join_kv_chunks(
-            *lists, q_entries, req_entries, req_offs, req_lens, meta.phase_node_nums, meta.phase_node_offsets,
-            meta.kv_group_num, meta.num_kv_heads, return_order=True)
-        req_entries, req_offs, req_lens = req_entries[: int(np.sum(req_lens))].tolist(), req_offs.tolist(), req_lens.tolist()
-        # a request's last vnode is the single-request vnode that ends where its tokens end; when
-        # that one went with a chunk, the vnode its chain was given to ends there now
+        sched = block_programs(*lists, q_entries, len(batch.reqs), meta.kv_group_num, meta.num_kv_heads,
+                               head_dim=meta.head_dim)
+        lists = [x.tolist() for x in (sched.kv_offs, sched.kv_lens, sched.q_offs, sched.q_lens)]
+        q_entries = sched.q_entries.tolist()
+        req_entries = sched.req_entries[: sched.num_rows].tolist()
+        req_offs, req_lens = sched.req_offs.tolist(), sched.req_lens.tolist()
+        # a request's last vnode is the single-request vnode that ends where its tokens end
+        # (narrow vnodes keep the planner's chunks, so there is exactly one)
         ends_of = {}
-        for v, (ko, kl, qo, ql) in enumerate(zip(*(x.tolist() for x in lists))):
+        for v, (ko, kl, qo, ql) in enumerate(zip(*lists)):
             if ql == 1:
                 ends_of[(ko + kl, q_entries[qo])] = v
-        last = [int(kept[v]) if kept[v] >= 0 else ends_of[(end, rid)]
-                for rid, (v, end) in enumerate(zip(meta.req_last_vnodes, tail_ends))]
-        *arranged, nums, offs, where = vnodes_in_launch_order(
-            *lists, nums, offs, meta.kv_group_num, meta.num_kv_heads, q_tile=q_tiles[0], return_order=True)
-        lists = [x.tolist() for x in arranged]
-        meta.phase_node_nums, meta.phase_node_offsets = nums, offs
-        # (single-request vnodes of the second phase are never absorbed as query tiles)
-        meta.req_last_vnodes = [int(where[v]) for v in last]
+        meta.req_last_vnodes = [ends_of[(end, rid)] for rid, end in enumerate(tail_ends)]
+        nums = LaunchPhases(sched.phase_node_nums)
+        if sched.num_programs > 0:
+            table = sched.prog_table.reshape(-1)
+            if table.size > meta.prog_table.numel():
+                raise ValueError(f"{sched.num_programs} block programs do not fit the {meta.prog_table.numel() // 4} "
+                                 "that max_vnodes allows")
+            src = torch.from_numpy(np.ascontiguousarray(table))
+            meta.prog_table[: src.numel()].copy_(src, non_blocking=True)
+            nums.prog_table = meta.prog_table[: src.numel()]
+            nums.num_programs = sched.num_programs
+            nums.narrow_in_programs = sched.narrow_in_programs
+        meta.phase_node_nums, meta.phase_node_offsets = nums, list(sched.phase_node_offsets)
 
     def upload(dst, values):
         src = torch.tensor(values, device="cpu", dtype=torch.int32)
@@ -345,6 +355,16 @@ def annotate_function(owner, func_name):
 
     annotated.__wrapped__ = original
     setattr(owner, func_name, annotated)
+
+
+def same_requests(planned_for, reqs) -> bool:
+    """Whether ``reqs`` are, one by one, the very objects of ``planned_for`` (a tuple kept from
+    the batch the plan was made for, or None).  The tuple holds the request objects themselves,
+    so none of them can have been freed and its address given to a new request in between, which
+    a comparison of ``id()`` values could not rule out (plugin.py:213-231 re-plans whenever the
+    reference's batch object changes)."""
+    return (planned_for is not None and len(planned_for) == len(reqs)
+            and all(a is b for a, b in zip(planned_for, reqs)))
 
 
 def load_fasttree_plugin(enable_fasttree=True, annotate_breakdown=False):
@@ -424,12 +444,11 @@ def load_fasttree_plugin(enable_fasttree=True, annotate_breakdown=False):
     decode_batch = ModelTpServer.forward_decode_batch
 
     def decode_batch_with_plan(self, batch):
-        members = tuple(id(r) for r in batch.reqs)
-        if self._fasttree_planned_for == members:
+        if same_requests(self._fasttree_planned_for, batch.reqs):
             this.prepare_for_fasttree_step(batch, self.fasttree_metadata)
         else:
             this.prepare_for_fasttree_meta(batch, self.fasttree_metadata)
-            self._fasttree_planned_for = members
+            self._fasttree_planned_for = tuple(batch.reqs)
         return decode_batch(self, batch)
 
     ModelTpServer.forward_decode_batch = decode_batch_with_plan

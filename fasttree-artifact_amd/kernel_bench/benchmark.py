@@ -18,7 +18,9 @@ call, a repetition count sized for about 100 ms, the median reported in millisec
 the parallelism thresholds and of the KV split sizes with the ones for MI355X: tiles of 64 // g
 and 16 // g requests, as the reference's sweep picks them per GQA ratio
 (kernel_bench/run_benchmark.sh:46-53), thresholds for 256 compute units instead of 132, and KV
-splits of 1024,256 instead of 1024,128 tokens; explicit options win over it.
+splits of 1024,256 instead of 1024,128 tokens; explicit options win over it.  It also asks the
+planner for its lists arranged as block programs for the part (``launch_order=True``) instead of in
+the reference's order.
 """
 import argparse
 import os
@@ -140,7 +142,7 @@ def main(args):
         _planner.VERBOSE = not args.quiet
         fasttree_aux, node_assignment = fasttree_preparation(
             tree_info, KV_ptrs, batch_size, num_qo_heads, num_kv_heads, head_dim,
-            KV_SPLIT_SIZES, para_threshs1, para_threshs2, params)
+            KV_SPLIT_SIZES, para_threshs1, para_threshs2, params, launch_order=args.mi355x)
         if args.fasttree_heuristic_path:
             with open(args.fasttree_heuristic_path, "w") as file:
                 for i in range(len(tree_info)):
@@ -187,7 +189,8 @@ def build_parser():
     parser.add_argument("--choice", type=str, choices=["flash_attn", "fasttree", "all"], default="all")
     parser.add_argument("--profile", action="store_true", default=False)
     parser.add_argument("--mi355x", action="store_true", default=False,
-                        help="query tiles, parallelism thresholds and KV split sizes for MI355X instead of the H100 defaults")
+                        help="query tiles, parallelism thresholds and KV split sizes for MI355X instead of the H100 defaults, "
+                             "and the planner's lists arranged as block programs for the part")
     parser.add_argument("--quiet", action="store_true", default=False, help="do not print the planner's lines")
     return parser
 

@@ -118,6 +118,46 @@ int ft_decode(const void* q, const void* k, const void* v, void* o,
               float sm_scale, int dtype, ft_stream_t stream);
 
 /*
+ * Stage 1 of a launch that the host has arranged as block programs, and the whole decode call
+ * with it (then ft_stage2).  No counterpart in the reference, which leaves the order and the
+ * placement of its (vnode, KV head) blocks to the hardware dispatcher (kernel_bench/fasttree.py:
+ * 443-479, grid = (node_num, head_num)).  One thread block per program and KV head walks the
+ * program: prog_table holds four int32 per program in device memory -- first and end of its
+ * vnodes within the range [phase_node_offsets[0], + phase_node_nums[0]) (served one after the
+ * other, whole blocks), then first and count of its vnodes within the range
+ * [phase_node_offsets[1], + phase_node_nums[1]) (served one wave each; a negative count means
+ * before the others instead of after them).  The first narrow_in_programs vnodes of the second
+ * range belong to programs; the rest of it is served one wave each by blocks of their own, as in
+ * ft_stage1_phases, whatever their width.  The lists are otherwise those of ft_decode and
+ * describe a complete plan without the table.  head_dim in {32, 64, 128}.  The table is
+ * trusted: it is not read on the host.
+ */
+int ft_stage1_programs(const void* q, const void* k, const void* v,
+                       int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+                       const int32_t* vnode_to_kv_entries, const int32_t* vnode_to_kv_offs,
+                       const int32_t* vnode_to_kv_lens, const int32_t* vnode_to_q_entries,
+                       const int32_t* vnode_to_q_offs, const int32_t* vnode_to_q_lens,
+                       float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
+                       const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
+                       const int32_t* prog_table, int num_programs, int narrow_in_programs,
+                       int num_qo_heads, int num_kv_heads, int head_dim,
+                       float sm_scale, int dtype, ft_stream_t stream);
+
+int ft_decode_programs(const void* q, const void* k, const void* v, void* o,
+                       int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+                       int64_t oo0, int64_t oo1,
+                       const int32_t* vnode_to_kv_entries, const int32_t* vnode_to_kv_offs,
+                       const int32_t* vnode_to_kv_lens, const int32_t* vnode_to_q_entries,
+                       const int32_t* vnode_to_q_offs, const int32_t* vnode_to_q_lens,
+                       const int32_t* req_to_vnode_entries, const int32_t* req_to_vnode_offs,
+                       const int32_t* req_to_vnode_lens,
+                       float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
+                       const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
+                       const int32_t* prog_table, int num_programs, int narrow_in_programs,
+                       int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
+                       float sm_scale, int dtype, ft_stream_t stream);
+
+/*
  * Decode attention without prefix sharing over a per-request gathered, padded cache
  * k_cache, v_cache [batch, max_seqlen, Hkv, D] (contiguous) with cache_seqlens [batch]:
  * the layout the reference's comparison engines read (kernel_bench/flash_attn_wrap.py:36-70,

@@ -120,15 +120,15 @@ def test_baseline_configs_against_dense_oracle(name, preset, device):
     assert_parity(o, ref.reshape(batch, hq, 128), f"{name}/{preset} vs torch fp32")
 
 
-@pytest.mark.parametrize("spec,moves", [
-    ({"kind": "irregular", "seed": 3}, False),
-    ({"kind": "regular", "sizes": [1, 2, 4, 8, 16, 32, 64, 128, 1024], "lens": [16] * 9}, True),
-])
-def test_vnode_order_within_a_phase_does_not_change_the_result(spec, moves, device):
-    """The launch order of fasttree_preparation (second phase listed longest first; with more
-    first-phase blocks than the device runs at a time, light first-phase vnodes moved to the
-    second phase) against the planner's own order."""
-    _announce("vnode order", spec["kind"])
+@pytest.mark.parametrize("spec", [
+    {"kind": "irregular", "seed": 3},
+    {"kind": "regular", "sizes": [1, 2, 4, 8, 16, 32, 64, 128, 1024], "lens": [16] * 9},
+], ids=["irregular", "nine_levels_of_16_tokens"])
+def test_launch_order_does_not_change_the_result(spec, device):
+    """The lists of fasttree_preparation(launch_order=True) -- block programs, scratch rows and
+    per-request lists of their own, light first-phase vnodes served with the second phase --
+    against the planner's own lists, both through fasttree_decode."""
+    _announce("launch order", spec["kind"])
     tree, ptrs, batch = build_tree(spec)
     inp = make_decode_inputs(tree, 32, 8, 128, device=device, dtype=torch.float16, seed=11, shuffle_slots=True)
     outs = []
@@ -140,17 +140,15 @@ def test_vnode_order_within_a_phase_does_not_change_the_result(spec, moves, devi
                                       device=device, kv_slot_map=inp.slot_map, launch_order=launch_order)
         wide = aux[11][0]
         q_lens = aux[5].cpu().numpy()[wide:].astype(np.int64)
-        work = aux[2].cpu().numpy()[wide:].astype(np.int64) * ((q_lens * 4 + 15) // 16)
         if launch_order:
-            assert (np.diff(work) <= 0).all()
-            assert moves == bool((q_lens > 4).any()), "light first-phase vnodes run with the second phase"
+            assert getattr(aux[11], "num_programs", 0) > 0 or wide == 0
         else:
-            assert (q_lens <= 4).all()
+            assert type(aux[11]) is list and (q_lens <= 4).all()
         outs.append(_decode(inp.Q, inp.K_pool, inp.V_pool, aux, [16, 4], [32, 32], 1.0 / math.sqrt(128)))
-    # (not bit for bit: a light first-phase vnode is computed by the second phase's code path)
+    # (not bit for bit: runs are cut at other tokens, light vnodes go through the other code path)
     assert_parity(outs[1], outs[0].float(), "launch order vs planner order")
     for o in outs:
-        print(_dense_check(tree, inp, o, "vnode order", list(range(0, batch, 5 if batch < 600 else 37))), flush=True)
+        print(_dense_check(tree, inp, o, "launch order", list(range(0, batch, 5 if batch < 600 else 37))), flush=True)
 
 
 @pytest.mark.parametrize("seed", [0, 1, 2])
@@ -399,41 +397,73 @@ def test_wide_vnodes_in_row_chunks_and_uneven_tails(device):
 
 
 @pytest.mark.gpu
-def test_kv_chunks_joined_where_the_rows_fill_the_machine(device, monkeypatch):
-    """1 x 2048 shared tokens under 1024 requests, 32/8 heads: the launch order undoes the root's
-    KV split (4096 query rows fill the machine by themselves), two partial rows per request
-    instead of three; same result as with the planner's own lists, both at the parity bar.  Then
-    forced on a small three-level tree (every chain joined, dropped rows in the middle of the
-    scratch), fp16 and bf16."""
-    from fasttree_hip import planner
-    _announce("kv chunks joined")
+def test_runs_cut_anew_into_block_programs(device, monkeypatch):
+    """1 x 2048 shared tokens under 1024 requests, 32/8 heads: in launch order the root's run is
+    cut into equal programs (pieces at multiples of 64 tokens instead of the planner's two
+    chunks); same result as with the planner's own lists, both at the parity bar.  Then forced
+    on a small three-level tree (every run cut anew, every program of several vnodes), fp16 and
+    bf16, on all block slots and on half of them."""
+    from fasttree_hip import launch_schedule
+    _announce("block programs")
     sample = list(range(0, 1024, 41))
-    aux = _plan_and_check(device, [1, 1024], [2048, 32], 32, 8, 128, [16, 4], [1024, 256], "kv chunks joined",
+    aux = _plan_and_check(device, [1, 1024], [2048, 32], 32, 8, 128, [16, 4], [1024, 256], "block programs",
                           sample=sample, thr=((256, 1024), (256, 256)))
-    assert aux[8].tolist() == [2] * 1024 and aux[9].shape[0] == 3 * 1024 and max(aux[2].tolist()) == 2048
+    assert aux[11].num_programs > 0 and aux[9].shape[0] == aux[3].numel()
     ref = _plan_and_check(device, [1, 1024], [2048, 32], 32, 8, 128, [16, 4], [1024, 256], "kv chunks as planned",
                           sample=sample, thr=((256, 1024), (256, 256)), launch_order=False)
     assert ref[8].tolist() == [3] * 1024
-    monkeypatch.setattr(planner, "FULL_MACHINE_BLOCKS", 1)
-    for dtype in (torch.float16, torch.bfloat16):
-        aux = _plan_and_check(device, [1, 4, 36], [700, 300, 45], 16, 4, 128, [16, 4], [256, 64], f"kv chunks forced {dtype}",
-                              dtype=dtype, thr=((10**6, 10**6), (1, 1)))
-        ref = _plan_and_check(device, [1, 4, 36], [700, 300, 45], 16, 4, 128, [16, 4], [256, 64], f"kv chunks as planned {dtype}",
-                              dtype=dtype, thr=((10**6, 10**6), (1, 1)), launch_order=False)
-        assert max(ref[2].tolist()) <= 64 and max(aux[2].tolist()) == 1000 and max(aux[8].tolist()) <= 3 < min(ref[8].tolist())
+    aux = _plan_and_check(device, [1, 10, 400], [4000, 400, 40], 32, 8, 128, [16, 4], [1024, 256], "programs of several vnodes",
+                          sample=list(range(0, 400, 13)), thr=((256, 1024), (256, 256)))
+    table = aux[11].prog_table.cpu().view(-1, 4)
+    assert int((table[:, 1] - table[:, 0]).max()) > 1, "programs of several vnodes"
+    monkeypatch.setattr(launch_schedule, "MIN_PROGRAM_TILES", 0.0)
+    monkeypatch.setattr(launch_schedule, "MIN_PIECE_TOKENS", 64)
+    for slots in (512, 256, 4):
+        monkeypatch.setattr(launch_schedule, "BLOCK_SLOTS", slots)
+        for dtype in (torch.float16, torch.bfloat16):
+            aux = _plan_and_check(device, [1, 4, 36], [700, 300, 45], 16, 4, 128, [16, 4], [256, 64],
+                                  f"programs forced {slots} {dtype}", dtype=dtype, thr=((10**6, 10**6), (1, 1)))
+            table = aux[11].prog_table.cpu().view(-1, 4)
+            assert aux[11].num_programs > 0 and int(table[-1, 1]) == aux[11][0]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+def test_narrow_vnodes_inside_block_programs(dtype, device, monkeypatch):
+    """The narrow vnodes dealt to the programs (block_programs(embed=True)): served by the
+    program's waves before its wide vnodes (first half of a round of programs) or after them,
+    on C3-like and irregular trees, incl. programs with more narrow vnodes than waves and
+    programs without any."""
+    import functools
+    from fasttree_hip import launch_schedule, planner as planner_module
+    _announce("narrow vnodes in programs", dtype)
+    monkeypatch.setattr(launch_schedule, "MIN_PROGRAM_TILES", 0.0)
+    forced = functools.partial(launch_schedule.block_programs, embed=True, recut=True)
+    monkeypatch.setattr(launch_schedule, "block_programs", forced)
+    for sizes, lens, hq, hkv, q_tiles in (([1, 5, 200], [1500, 200, 40], 32, 8, [16, 4]),
+                                          ([1, 3, 37], [300, 100, 70], 16, 4, [16, 4]),
+                                          ([1, 700], [256, 33], 8, 8, [64, 16])):
+        aux = _plan_and_check(device, sizes, lens, hq, hkv, 128, q_tiles, [1024, 256], f"narrow in programs {sizes}",
+                              dtype=dtype, thr=((256, 1024), (256, 256)), sample=list(range(0, sizes[-1], 7)))
+        nums = aux[11]
+        table = nums.prog_table.cpu().view(-1, 4)
+        assert nums.narrow_in_programs == nums[1] > 0 and int(table[:, 3].abs().sum()) == nums[1]
+        assert bool((table[:, 3] < 0).any())
+        if sizes[-1] == 200:
+            assert bool((table[:, 3] > 0).any()), "some programs end with their narrow vnodes"
 
 
 @pytest.mark.gpu
 def test_more_wide_vnodes_than_the_ranking_holds(device):
     """More than 256 wide vnodes: blocks take them in plan order instead of ranking them (the
-    planner's own list; in launch order these light vnodes all run with the narrow phase)."""
+    planner's own list; in launch order the light ones among them run with the narrow phase)."""
     _announce("many wide vnodes")
     aux = _plan_and_check(device, [1, 300, 1800], [40, 70, 9], 32, 8, 128, [16, 4], [1024, 128], "many wide vnodes",
                           sample=list(range(0, 1800, 37)), launch_order=False)
     assert aux[11][0] > 256
     aux = _plan_and_check(device, [1, 300, 1800], [40, 70, 9], 32, 8, 128, [16, 4], [1024, 128], "many light vnodes",
                           sample=list(range(0, 1800, 37)))
-    assert aux[11][0] == 0
+    assert aux[11][0] < 256 and int(aux[5][aux[11][0]:].max()) * 4 > 16, "the light ones are served narrow"
 
 
 @pytest.mark.gpu
@@ -441,12 +471,12 @@ def test_more_wide_vnodes_than_the_ranking_holds(device):
 def test_light_wide_vnodes_run_with_the_narrow_phase_at_every_head_size(d, device):
     """More first-phase blocks than the device holds, all of them light (32-64 rows x 20-30
     tokens): the launch order hands them to the narrow path, which serves them in passes of 16
-    rows (head_dim 256 goes through the register-staged kernel)."""
+    rows (head_dim 256 goes through the register-staged kernel, without the program table)."""
     _announce("light wide vnodes", d)
     aux = _plan_and_check(device, [1, 150, 1200], [20, 30, 9], 16, 4, d, [16, 4], [1024, 128], f"light wide d{d}",
                           sample=list(range(0, 1200, 23)), thr=((132, 528), (132, 132)))
     wide = aux[11][0]
-    assert wide == 0 and int(aux[5].max()) * 4 > 16, "every vnode is launched narrow, some with more than 16 rows"
+    assert wide < 225 and int(aux[5][wide:].max()) * 4 > 16, "the light vnodes are launched narrow, with more than 16 rows"
     aux = _plan_and_check(device, [1, 150, 1200], [20, 30, 9], 16, 4, d, [16, 4], [1024, 128], f"light wide d{d}, planner order",
                           sample=list(range(0, 1200, 23)), thr=((132, 528), (132, 132)), launch_order=False)
     assert aux[11][0] == 225

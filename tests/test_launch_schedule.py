@@ -1,0 +1,179 @@
+"""The launch schedule of the first decode stage (block programs), on the CPU: whatever the
+arrangement, every request attends every token of its path exactly once, through scratch rows
+that are listed for it; the program table describes the lists it comes with."""
+
+import numpy as np
+import pytest
+
+from cases import PLANNER_CASES, build_tree
+from fasttree_hip import launch_schedule as ls
+from fasttree_hip.launch_schedule import LaunchPhases, block_programs
+from helpers import run_planner
+
+NAMES = ["kat1", "c1", "c3", "c5_seed0", "c5_seed1", "shape07_h32_8", "shape07_h16_1_gamma10", "rand03", "rand17", "rand41"]
+VARIANTS = {
+    "default": {},
+    "cut_anew": dict(recut=True),
+    "planner_chunks": dict(recut=False),
+    "narrow_in_programs": dict(recut=True, embed=True),
+    "narrow_in_programs_auto": dict(embed=None),
+    "one_block_per_unit": dict(block_slots=256),
+    "two_blocks_per_unit": dict(block_slots=512, recut=True),
+}
+
+
+def _attended(kv_offs, kv_lens, q_offs, q_lens, q_entries, req_entries, req_offs, req_lens, batch):
+    """For each request: the KV index entries the scratch rows *listed for it* attend."""
+    row_vnode = {}
+    for v, (qo, ql) in enumerate(zip(q_offs, q_lens)):
+        for i in range(ql):
+            assert qo + i not in row_vnode, "a scratch row belongs to at most one vnode"
+            row_vnode[qo + i] = v
+    assert sorted(row_vnode) == list(range(len(q_entries))), "every scratch row belongs to a vnode"
+    seen = []
+    for r in range(batch):
+        rows = list(req_entries[req_offs[r]: req_offs[r] + req_lens[r]])
+        assert rows == sorted(set(rows)) and all(q_entries[x] == r for x in rows)
+        got = []
+        for x in rows:
+            v = row_vnode[x]
+            got.extend(range(kv_offs[v], kv_offs[v] + kv_lens[v]))
+        seen.append(sorted(got))
+    assert sum(req_lens[:batch]) == len(q_entries), "every scratch row is listed for its request"
+    return seen
+
+
+def _plan_lists(plan):
+    return (plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens, plan.vnode_to_q_entries)
+
+
+def _schedule(case, **kw):
+    tree, ptrs, batch, plan, params, _ = run_planner(case)
+    group = case["Hq"] // case["Hkv"]
+    sched = block_programs(*_plan_lists(plan), batch, group, case["Hkv"], **kw)
+    return plan, batch, group, sched
+
+
+@pytest.mark.parametrize("variant", list(VARIANTS))
+@pytest.mark.parametrize("name", NAMES)
+def test_every_request_still_attends_its_path_once(name, variant):
+    case = next(c for c in PLANNER_CASES if c["name"] == name)
+    plan, batch, group, s = _schedule(case, **VARIANTS[variant])
+    before = _attended(*_plan_lists(plan), plan.req_to_vnode_entries, plan.req_to_vnode_offs, plan.req_to_vnode_lens, batch)
+    after = _attended(s.kv_offs.tolist(), s.kv_lens.tolist(), s.q_offs.tolist(), s.q_lens.tolist(), s.q_entries.tolist(),
+                      s.req_entries.tolist(), s.req_offs.tolist(), s.req_lens.tolist(), batch)
+    assert after == before
+    # the per-request lists end with the reference's padding (kernel_bench/fasttree.py:261-262)
+    assert s.req_entries[-32:].tolist() == [-1] * 32 and len(s.req_entries) == s.num_rows + 32
+    # phases: the programs' vnodes first, then the vnodes served one wave each
+    n_wide, n_narrow = s.phase_node_nums
+    assert s.phase_node_offsets == [0, n_wide] and n_wide + n_narrow == len(s.kv_offs)
+    assert (s.q_lens[:n_wide] * group <= ls.BLOCK_ROWS).all(), "a program's vnode fits one pass of a block"
+    assert (s.kv_lens > 0).all()
+
+
+@pytest.mark.parametrize("variant", list(VARIANTS))
+@pytest.mark.parametrize("name", NAMES)
+def test_program_table_describes_the_lists(name, variant):
+    case = next(c for c in PLANNER_CASES if c["name"] == name)
+    _, _, _, s = _schedule(case, **VARIANTS[variant])
+    t = s.prog_table
+    n_wide, n_narrow = s.phase_node_nums
+    assert t.shape == (s.num_programs, 4) and t.dtype == np.int32
+    if n_wide == 0:
+        assert s.num_programs == 0 and s.narrow_in_programs == 0
+        return
+    # every wide vnode belongs to exactly one program, in order, and no program is empty
+    assert t[0, 0] == 0 and t[-1, 1] == n_wide
+    assert (t[1:, 0] == t[:-1, 1]).all() and (t[:, 1] > t[:, 0]).all()
+    # the programs' narrow vnodes lie back to back at the head of the second phase
+    counts = np.abs(t[:, 3])
+    assert (t[:, 2] == np.concatenate([[0], np.cumsum(counts)[:-1]])).all()
+    assert counts.sum() == s.narrow_in_programs <= n_narrow
+    if not VARIANTS[variant].get("embed", False):
+        assert s.narrow_in_programs == 0 or VARIANTS[variant].get("embed", False) is None
+    assert len(s.program_tiles) == s.num_programs and (s.program_tiles > 0).all()
+    assert s.modelled_us > 0
+
+
+def test_headline_tree_is_cut_into_equal_programs():
+    """C3 (3-level tree, 400 requests, 32/8 heads): the 4000-token root under 1600 query rows and
+    the ten 400-token nodes under 160 rows become at most 64 programs per kv head (512 block
+    slots / 8 heads) whose modelled work differs by a few percent; pieces start and end at
+    multiples of 64 tokens of their run; the 400 leaves stay as the planner made them."""
+    case = next(c for c in PLANNER_CASES if c["name"] == "c3")
+    plan, batch, group, s = _schedule(case, block_slots=512)
+    assert 56 <= s.num_programs <= 64
+    assert s.program_tiles.max() <= 1.1 * s.program_tiles.mean()
+    n_wide, n_narrow = s.phase_node_nums
+    assert n_narrow == 400 and sorted(s.kv_lens[n_wide:].tolist()) == [40] * 400 and set(s.q_lens[n_wide:].tolist()) == {1}
+    root = [(int(o), int(n)) for o, n in zip(s.kv_offs[:n_wide], s.kv_lens[:n_wide]) if o < 4000]
+    assert all(o % ls.CUT_TOKENS == 0 for o, _ in root) and all(n >= ls.MIN_PIECE_TOKENS for _, n in root)
+    # every row chunk of the root covers its 4000 tokens once
+    by_rows = {}
+    for v in range(n_wide):
+        if s.kv_offs[v] < 4000:
+            by_rows.setdefault(int(s.q_entries[s.q_offs[v]]), []).append((int(s.kv_offs[v]), int(s.kv_lens[v])))
+    assert len(by_rows) == 13   # 1600 rows in 13 even chunks of at most 128
+    for pieces in by_rows.values():
+        pieces.sort()
+        assert pieces[0][0] == 0 and sum(n for _, n in pieces) == 4000
+        assert all(a + n == b for (a, n), (b, _) in zip(pieces, pieces[1:]))
+
+
+def test_small_launches_keep_the_planner_chunks():
+    """A launch whose programs would hold less than MIN_PROGRAM_TILES keeps the planner's KV
+    chunks, one vnode per program, longest first; a launch without wide vnodes has no programs."""
+    case = next(c for c in PLANNER_CASES if c["name"] == "c1")
+    plan, batch, group, s = _schedule(case)
+    assert s.num_programs == 0 and s.phase_node_nums == [0, len(plan.vnode_to_kv_offs)]
+    assert sorted(zip(s.kv_offs.tolist(), s.kv_lens.tolist())) == sorted(zip(plan.vnode_to_kv_offs, plan.vnode_to_kv_lens))
+    tree, ptrs, batch = build_tree({"kind": "regular", "sizes": [1, 64], "lens": [512, 32]})
+    from fasttree_hip.planner import FastTreeParams, fasttree_plan
+    p = FastTreeParams(); p.set_values(0.66, 0.33, 0.1); p.set_q_tile_sizes([16, 4]); p.set_kv_tile_sizes([32, 32]); p.set_kv_group_num(4)
+    plan = fasttree_plan(tree, ptrs, batch, 8, [256, 256], [1, 1], [1, 1], p)
+    assert plan.phase_node_nums[0] == 8
+    s = block_programs(*_plan_lists(plan), batch, 4, 8)
+    n_wide = s.phase_node_nums[0]
+    assert s.num_programs == n_wide > 0 and (s.prog_table[:, 1] - s.prog_table[:, 0] == 1).all()
+    chunk_lens = sorted(set(plan.vnode_to_kv_lens[: plan.phase_node_nums[0]]))
+    assert sorted(set(s.kv_lens[:n_wide].tolist())) == chunk_lens
+    assert (np.diff(s.program_tiles) <= 0).all()
+
+
+def test_narrow_vnodes_dealt_to_programs_in_equal_shares():
+    """With embed=True every program gets its share of the narrow vnodes (counts differ by at
+    most one), the two halves of a round of programs in opposite orders (negative count: before
+    the wide vnodes)."""
+    case = next(c for c in PLANNER_CASES if c["name"] == "c3")
+    _, _, _, s = _schedule(case, recut=True, embed=True, block_slots=512)
+    counts = np.abs(s.prog_table[:, 3])
+    assert s.narrow_in_programs == 400 == counts.sum() and counts.max() - counts.min() <= 1
+    per_round = 512 // 8
+    front = s.prog_table[:, 3] < 0
+    assert front[: per_round // 2].all() and not front[per_round // 2: per_round].any()
+
+
+def test_preparation_in_launch_order_carries_the_programs():
+    """fasttree_preparation(launch_order=True): the phase list is a list of two counts that also
+    carries the program table (a device tensor) -- with and without preallocated buffers."""
+    import torch
+    from fasttree_hip.planner import FastTreeParams, PlanBuffers, fasttree_preparation
+    case = next(c for c in PLANNER_CASES if c["name"] == "c3")
+    tree, ptrs, batch = build_tree(case["tree"])
+    buffers = PlanBuffers(32, 128, max_kv_entries=400000, max_rows=8192, max_vnodes=8192, max_batch_size=2048, device="cpu")
+    outs = []
+    for buf in (None, buffers):
+        p = FastTreeParams(); p.set_values(0.66, 0.33, 0.1); p.set_q_tile_sizes([16, 4]); p.set_kv_tile_sizes([32, 32]); p.set_kv_group_num(4)
+        aux, _ = fasttree_preparation(tree, ptrs, batch, 32, 8, 128, [1024, 256], [256, 1024], [256, 256], p,
+                                      device="cpu", launch_order=True, buffers=buf)
+        nums = aux[11]
+        assert isinstance(nums, LaunchPhases) and isinstance(nums, list) and len(nums) == 2 and aux[12] == [0, nums[0]]
+        assert nums.prog_table.dtype == torch.int32 and nums.prog_table.numel() == 4 * nums.num_programs > 0
+        assert int(nums.prog_table.view(-1, 4)[-1, 1]) == nums[0] and nums.narrow_in_programs == 0
+        assert aux[9].shape[0] == aux[3].numel() == int(aux[8].sum())
+        outs.append(aux)
+    for a, b in zip(outs[0][:9], outs[1][:9]):
+        assert torch.equal(a, b)
+    assert torch.equal(outs[0][11].prog_table, outs[1][11].prog_table)
+    assert outs[1][11].prog_table.data_ptr() == buffers.prog_table.data_ptr()

@@ -130,211 +130,35 @@ def test_plan_invariants(name):
         assert rows == sorted(rows) and all(plan.vnode_to_q_entries[x] == r for x in rows)
 
 
-@pytest.mark.parametrize("light_work", [0, 4096, 1 << 40])
-@pytest.mark.parametrize("name", ["kat1", "c3", "c5_seed0", "rand17", "shape07_h32_8"])
-def test_launch_order_is_a_permutation_of_the_vnodes(name, light_work):
-    """The launch order keeps the vnode tuples; first-phase vnodes of at most light_work rows x
-    tokens join the second phase, which is listed by decreasing tokens x passes with ties in the
-    previous order; the other first-phase vnodes keep their order."""
-    from fasttree_hip.planner import vnodes_in_launch_order
-    case = next(c for c in PLANNER_CASES if c["name"] == name)
-    tree, ptrs, batch, plan, params, _ = run_planner(case)
-    group = case["Hq"] // case["Hkv"]
-    before = list(zip(plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens))
-    *lists, nums, offs = vnodes_in_launch_order(
-        plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens,
-        plan.phase_node_nums, plan.phase_node_offsets, group, light_work=light_work)
-    after = list(zip(*(x.tolist() for x in lists)))
-    wide = plan.phase_node_nums[0]
-    light = lambda v: v[1] * v[3] * group <= light_work and v[3] * group <= 64
-    work = lambda v: v[1] * ((v[3] * group + 15) // 16)
-    stay = [v for v in before[:wide] if not light(v)]
-    move = [v for v in before[:wide] if light(v)]
-    assert nums == [len(stay), len(before) - len(stay)] and offs == [0, len(stay)]
-    assert after[:nums[0]] == stay
-    assert after[nums[0]:] == sorted(move + before[wide:], key=lambda v: -work(v))  # (sorted() is stable)
-    assert sorted(after) == sorted(before)
-    assert list(plan.vnode_to_kv_lens) == [v[1] for v in before], "the plan itself is not touched"
-    if light_work == 0:
-        assert nums == list(plan.phase_node_nums)
-    # with the number of kv heads given, nothing moves unless the first phase oversubscribes the machine
-    *_, nums_few, _ = vnodes_in_launch_order(
-        plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens,
-        plan.phase_node_nums, plan.phase_node_offsets, group, 1, light_work=light_work)
-    assert nums_few == (nums if wide > 512 else list(plan.phase_node_nums))
-
-
-@pytest.mark.parametrize("name", ["c3", "c5_seed0", "shape07_h32_8", "rand17", "rand41"])
-def test_launch_order_joins_query_tiles_without_changing_what_is_computed(name):
-    """With the query tile given, neighbouring tiles of one run become one vnode of at most 128
-    rows x chunks: every (run, scratch row) pair is still served exactly once."""
-    from fasttree_hip.planner import vnodes_in_launch_order
-    case = next(c for c in PLANNER_CASES if c["name"] == name)
-    tree, ptrs, batch, plan, params, _ = run_planner(case)
-    group = case["Hq"] // case["Hkv"]
-
-    def pairs(kv_offs, kv_lens, q_offs, q_lens):
-        out = []
-        for ko, kl, qo, ql in zip(kv_offs, kv_lens, q_offs, q_lens):
-            out.extend((int(ko), int(kl), int(qo) + i) for i in range(int(ql)))
-        return sorted(out)
-
-    before = pairs(plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens)
-    q_tile = plan.q_tile_sizes[0]
-    *lists, nums, offs = vnodes_in_launch_order(
-        plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens,
-        plan.phase_node_nums, plan.phase_node_offsets, group, None, light_work=0, q_tile=q_tile)
-    assert pairs(*lists) == before
-    assert len(set(p[2] for p in before)) == plan.num_rows == len(before)
-    chunks = max(1, min(8, -(-q_tile * group // 128)))
-    cap = 128 * chunks // group
-    wide_q = lists[3][:nums[0]]
-    assert nums[1] == plan.phase_node_nums[1] and nums[0] <= plan.phase_node_nums[0] and offs == [0, nums[0]]
-    assert all(q <= max(cap, q_tile) for q in wide_q)
-    # no two neighbours left that could still be joined
-    for v in range(1, nums[0]):
-        same = lists[0][v] == lists[0][v - 1] and lists[1][v] == lists[1][v - 1] and lists[2][v - 1] + lists[3][v - 1] == lists[2][v]
-        assert not (same and lists[3][v - 1] + lists[3][v] <= cap)
-    if name == "c3":
-        # 100 root tiles of 16 requests in 4 splits -> 13 per split; 10 x (16, 16, 8) -> 10 x (32, 8)
-        assert plan.phase_node_nums[0] == 130 and nums[0] == 4 * 13 + 10 * 2
-    # with the kv heads given and no more blocks than compute units, nothing is joined
-    *_, nums_few, _ = vnodes_in_launch_order(
-        plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens,
-        plan.phase_node_nums, plan.phase_node_offsets, group, 1, light_work=0, q_tile=q_tile)
-    if 2 * plan.phase_node_nums[0] * chunks <= 512:
-        assert nums_few == list(plan.phase_node_nums)
-
-
-def _joined_plan(plan, group, hkv, min_blocks):
-    """`plan` with its vnode and per-request lists replaced by what join_kv_chunks returns."""
-    import copy
-    from fasttree_hip.planner import join_kv_chunks
-    out = join_kv_chunks(plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens,
-                         plan.vnode_to_q_entries, plan.req_to_vnode_entries, plan.req_to_vnode_offs, plan.req_to_vnode_lens,
-                         plan.phase_node_nums, plan.phase_node_offsets, group, hkv, min_blocks=min_blocks)
-    new = copy.copy(plan)
-    (new.vnode_to_kv_offs, new.vnode_to_kv_lens, new.vnode_to_q_offs, new.vnode_to_q_lens,
-     new.req_to_vnode_entries, new.req_to_vnode_offs, new.req_to_vnode_lens) = (x.tolist() for x in out[:7])
-    new.phase_node_nums, new.phase_node_offsets = out[7], out[8]
-    return new
-
-
-def _attended(plan, batch):
-    """For each request: the KV index entries the scratch rows *listed for it* attend."""
-    row_vnode = {}
-    for v, (qo, ql) in enumerate(zip(plan.vnode_to_q_offs, plan.vnode_to_q_lens)):
-        for i in range(ql):
-            assert qo + i not in row_vnode, "a scratch row belongs to at most one vnode"
-            row_vnode[qo + i] = v
-    seen = []
-    for r in range(batch):
-        rows = plan.req_to_vnode_entries[plan.req_to_vnode_offs[r]: plan.req_to_vnode_offs[r] + plan.req_to_vnode_lens[r]]
-        assert rows == sorted(set(rows)) and all(plan.vnode_to_q_entries[x] == r for x in rows)
-        got = []
-        for x in rows:
-            v = row_vnode[x]
-            got.extend(range(plan.vnode_to_kv_offs[v], plan.vnode_to_kv_offs[v] + plan.vnode_to_kv_lens[v]))
-        seen.append(sorted(got))
-    assert sorted(row_vnode) == sorted(x for r in range(batch) for x in
-                                       plan.req_to_vnode_entries[plan.req_to_vnode_offs[r]: plan.req_to_vnode_offs[r] + plan.req_to_vnode_lens[r]]), \
-        "every row of a kept vnode is listed for its request, and no dropped row is"
-    return seen
-
-
-@pytest.mark.parametrize("name", ["kat1", "c3", "c5_seed0", "c5_seed1", "shape07_h32_8", "rand03", "rand17", "rand41"])
-def test_joining_kv_chunks_keeps_what_every_request_attends(name):
-    """Forced (one block is enough): every chain of chunks is joined; each request still attends
-    the same entries of the flat KV list, each once, through the rows listed for it; the joined
-    vnodes keep phase and tile widths; the trailing 32 x -1 are there."""
-    case = next(c for c in PLANNER_CASES if c["name"] == name)
-    tree, ptrs, batch, plan, params, _ = run_planner(case)
-    group = case["Hq"] // case["Hkv"]
-    before = _attended(plan, batch)
-    new = _joined_plan(plan, group, case["Hkv"], min_blocks=1)
-    assert _attended(new, batch) == before
-    assert new.req_to_vnode_entries[-32:] == [-1] * 32 and len(new.req_to_vnode_entries) == sum(new.req_to_vnode_lens) + 32
-    wide = new.phase_node_nums[0]
-    assert new.phase_node_offsets == [0, wide] and sum(new.phase_node_nums) == len(new.vnode_to_kv_offs)
-    assert all(n > plan.q_tile_sizes[1] for n in new.vnode_to_q_lens[:wide])
-    assert all(n <= plan.q_tile_sizes[1] for n in new.vnode_to_q_lens[wide:])
-    # nothing left to join: no run (the vnodes over one KV slice) is followed by a run over the same requests in the same tiles
-    runs = {}
-    for ko, kl, qo, ql in zip(new.vnode_to_kv_offs, new.vnode_to_kv_lens, new.vnode_to_q_offs, new.vnode_to_q_lens):
-        runs.setdefault((ko, kl), []).append(tuple(new.vnode_to_q_entries[qo: qo + ql]))
-    for (ko, kl), tiles in runs.items():
-        for (ko2, kl2), tiles2 in runs.items():
-            assert not (ko2 == ko + kl and tiles2 == tiles)
-    if name == "c3":
-        # the root's four chunks become one per query tile: 100 + 30 -> 25 + 30 first-phase vnodes, 3 rows fewer per request
-        assert plan.phase_node_nums == [130, 400] and new.phase_node_nums == [55, 400]
-        assert set(new.req_to_vnode_lens) == {3} and set(plan.req_to_vnode_lens) == {6}
-    # the inputs are untouched; with the default thresholds small trees stay as they are, and C3's root gets three
-    # chunks of 1344, 1344 and 1312 tokens instead of four (3 x 104 + 160 = 472 first-phase blocks instead of 576)
-    same = _joined_plan(plan, group, case["Hkv"], min_blocks=None)
-    assert _attended(same, batch) == before
-    if name == "c3":
-        assert same.phase_node_nums == [3 * 25 + 30, 400] and set(same.req_to_vnode_lens) == {5}
-        assert sorted(set(same.vnode_to_kv_lens[:75])) == [1312, 1344] and same.vnode_to_kv_offs[50] == 2688
-    elif name not in ("c5_seed0", "c5_seed1"):
-        assert same.vnode_to_kv_lens == list(plan.vnode_to_kv_lens) and same.req_to_vnode_entries == list(plan.req_to_vnode_entries)
-
-
-def test_kv_chunks_are_cut_anew_to_fit_the_first_phase_into_the_machine():
-    """C3 (root: 104 blocks per chunk, four chunks; the level below: 160 blocks): the root is cut
-    at the shortest chunk length that brings the first phase under the number of resident
-    blocks, as long as its own blocks still number nine tenths of `min_blocks`; else it keeps its four chunks."""
-    from fasttree_hip.planner import join_kv_chunks
-    case = next(c for c in PLANNER_CASES if c["name"] == "c3")
-    tree, ptrs, batch, plan, params, _ = run_planner(case)
-    before = _attended(plan, batch)
-    expectations = [(None, 10**9, 4), (None, 576, 4), (None, 575, 3), (None, 472, 3), (None, 471, 4),  # two chunks: 208 blocks < 230 = 9/10 x 256
-                    (232, 471, 2), (233, 471, 4), (105, 368, 2), (105, 367, 1), (105, 264, 1), (105, 263, 4),
-                    (104, 10**9, 1)]                                                                   # (104: the root alone fills the machine)
-    for min_blocks, resident, chunks in expectations:
-        out = join_kv_chunks(plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens,
-                             plan.vnode_to_q_entries, plan.req_to_vnode_entries, plan.req_to_vnode_offs, plan.req_to_vnode_lens,
-                             plan.phase_node_nums, plan.phase_node_offsets, 4, 8, min_blocks=min_blocks, resident_blocks=resident)
-        assert out[7] == [25 * chunks + 30, 400], (min_blocks, resident, out[7])
-        assert set(out[6].tolist()) == {chunks + 2}
-        root = sorted(set(zip(out[0][:25 * chunks].tolist(), out[1][:25 * chunks].tolist())))
-        assert len(root) == chunks and root[0][0] == 0 and sum(n for _, n in root) == 4000
-        assert all(a + n == b for (a, n), (b, _) in zip(root, root[1:])) and all(n % 64 == 0 for _, n in root[:-1])
-    new = _joined_plan(plan, 4, 8, None)
-    assert _attended(new, batch) == before
-
-
-def test_many_equal_chains_are_not_cut_into_a_few_long_blocks():
-    """16 nodes of 1500 tokens under a 3000-token root that the planner merges into them: 16
-    runs of 4500 tokens in five chunks, 8 blocks per chunk -- 640 blocks.  No run covers the
-    machine by itself, so none is cut anew (one chunk of 4500 tokens for some of them would be
-    what the launch waits for)."""
-    from fasttree_hip.planner import FastTreeParams, fasttree_plan
-    tree, ptrs, batch = build_tree({"kind": "regular", "sizes": [1, 16, 256], "lens": [3000, 1500, 100]})
-    p = FastTreeParams(); p.set_values(0.66, 0.33, 0.1); p.set_q_tile_sizes([16, 4]); p.set_kv_tile_sizes([32, 32]); p.set_kv_group_num(4)
-    plan = fasttree_plan(tree, ptrs, batch, 8, [1024, 256], [256, 1024], [256, 256], p)
-    assert plan.phase_node_nums == [80, 256] and max(plan.vnode_to_kv_lens) == 1024
-    new = _joined_plan(plan, 4, 8, None)
-    assert new.phase_node_nums == [80, 256] and new.vnode_to_kv_lens == list(plan.vnode_to_kv_lens)
-
-
-def test_joining_kv_chunks_only_where_the_rows_fill_the_machine():
-    """1 x 2048 shared tokens under 1024 requests, 32/8 heads: 4096 query rows = 32 blocks x 8 kv
-    heads = 256 blocks without the split, so the root's two chunks are joined; under 256 requests
-    (64 blocks) they are not."""
-    from fasttree_hip.planner import FastTreeParams, fasttree_plan
-    for leaves, joins in ((1024, True), (256, False)):
-        tree, ptrs, batch = build_tree({"kind": "regular", "sizes": [1, leaves], "lens": [2048, 32]})
-        p = FastTreeParams(); p.set_values(0.66, 0.33, 0.1); p.set_q_tile_sizes([16, 4]); p.set_kv_tile_sizes([32, 32]); p.set_kv_group_num(4)
-        plan = fasttree_plan(tree, ptrs, batch, 8, [1024, 256], [256, 1024], [256, 256], p)
-        assert plan.phase_node_nums == [2 * leaves // 16, leaves] and set(plan.req_to_vnode_lens) == {3}
-        new = _joined_plan(plan, 4, 8, None)
-        if joins:
-            assert new.phase_node_nums == [leaves // 16, leaves] and set(new.req_to_vnode_lens) == {2}
-            assert set(new.vnode_to_kv_lens[:leaves // 16]) == {2048}
-        else:
-            assert new.phase_node_nums == plan.phase_node_nums and new.vnode_to_kv_lens == list(plan.vnode_to_kv_lens)
-        assert _attended(new, batch) == _attended(plan, batch)
+@pytest.mark.parametrize("case", PLANNER_CASES, ids=[c["name"] for c in PLANNER_CASES])
+def test_preparation_returns_the_reference_lists_by_default(case, goldens):
+    """The function that carries the reference's name, called as the reference is (no
+    launch-order argument; `device` only because there is no GPU here), returns the reference's
+    tuple: the nine index arrays, scratch of the reference's shapes, the two phase lists as plain
+    lists, the assignments; it mutates `params` and prints as the reference does
+    (kernel_bench/fasttree.py:99-296)."""
+    import contextlib, io
+    import torch
+    from fasttree_hip.planner import fasttree_preparation
+    gold = goldens[case["name"]]
+    tree, ptrs, batch = build_tree(case["tree"])
+    params = params_for(case)
+    out = io.StringIO()
+    with contextlib.redirect_stdout(out):
+        aux, assignments = fasttree_preparation(tree, ptrs, batch, case["Hq"], case["Hkv"], case["D"],
+                                                list(case["kv_split_sizes"]), list(case["para_threshs1"]),
+                                                list(case["para_threshs2"]), params, device="cpu")
+    assert len(aux) == 13
+    for name, tensor in zip(ARRAYS[:9], aux[:9]):
+        assert tensor.dtype == torch.int32 and tensor.numel() == gold[name]["len"], name
+        assert digest(tensor.numpy()) == gold[name]["sha256"], name
+    assert digest(np.asarray(assignments, dtype=np.int32)) == gold["node_assignments"]["sha256"]
+    assert list(aux[9].shape) == gold["mid_o_shape"] and aux[9].dtype == torch.float32
+    assert list(aux[10].shape) == gold["mid_o_shape"][:2] and aux[10].dtype == torch.float32
+    assert type(aux[11]) is list and aux[11] == gold["phase_node_nums"]
+    assert type(aux[12]) is list and aux[12] == gold["phase_node_offsets"]
+    assert list(params.TSQs) == gold["final_TSQs"] and list(params.TSKs) == gold["final_TSKs"]
+    assert out.getvalue() == gold["stdout"]
 
 
 def test_preparation_into_preallocated_buffers():

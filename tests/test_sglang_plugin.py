@@ -130,21 +130,23 @@ def test_hand_derived_plan():
     assert got["req_offs"] == [0, 3, 6] and got["req_lens"] == [3, 3, 3]
     assert meta.req_last_vnodes == [3, 4, 5]
     assert batch.fasttree_metadata is meta
+    covered = [sorted(x) for x in covered_slots(meta, batch)]
     prepare_for_fasttree_step(batch, meta)
     assert meta.vnode_to_kv_lens[:6].tolist() == [4, 2, 3, 4, 3, 2]
 
-    # launch order (the default): the same vnodes, longest first within the phase; the tail
-    # vnodes are found at their new positions
+    # launch order (the default): the same vnodes with scratch rows of their own; the tail vnodes are found at their new positions
     meta2 = small_meta()
     prepare_for_fasttree_meta(batch, meta2)
     got2 = plan_lists(meta2, batch)
-    vnodes = lambda g: sorted(zip(g["kv_offs"], g["kv_lens"], g["q_offs"], g["q_lens"]))
+    vnodes = lambda g: sorted((o, n, tuple(g["q_entries"][qo:qo + ql]))
+                              for o, n, qo, ql in zip(g["kv_offs"], g["kv_lens"], g["q_offs"], g["q_lens"]))
     assert vnodes(got2) == vnodes(got) and list(meta2.phase_node_nums) == [0, 6]
-    assert got2["kv_lens"] == [4, 3, 3, 2, 2, 1]
-    for key in ("q_entries", "req_entries", "req_offs", "req_lens"):
-        assert got2[key] == got[key]
+    assert [sorted(x) for x in covered_slots(meta2, batch)] == covered
+    for r in range(3):
+        rows = got2["req_entries"][got2["req_offs"][r]: got2["req_offs"][r] + got2["req_lens"][r]]
+        assert len(rows) == 3 and all(got2["q_entries"][x] == r for x in rows)
     for r, v in enumerate(meta2.req_last_vnodes):
-        assert (got2["kv_offs"][v], got2["q_offs"][v]) == (got["kv_offs"][[3, 4, 5][r]], got["q_offs"][[3, 4, 5][r]])
+        assert got2["kv_offs"][v] == got["kv_offs"][[3, 4, 5][r]] and got2["q_entries"][got2["q_offs"][v]] == r
     prepare_for_fasttree_step(batch, meta2)
     assert sorted(meta2.vnode_to_kv_lens[:6].tolist()) == sorted([4, 2, 3, 4, 3, 2])
 
@@ -195,7 +197,7 @@ def test_chunk_joins_keep_the_coverage_and_the_last_vnodes(seed, monkeypatch):
     prompts and generated tails all longer than the KV split): every request still attends each
     of its tokens once through the rows listed for it, its last vnode is a single-request vnode
     that ends where its tokens end, and the in-place step makes it cover the next token."""
-    from fasttree_hip import planner
+    from fasttree_hip import launch_schedule
     rng = random.Random(100 + seed)
     system = [rng.randint(1, 10**6) for _ in range(rng.randint(20, 60))]
     prefixes, prompts, outputs = [system], [], []
@@ -208,7 +210,7 @@ def test_chunk_joins_keep_the_coverage_and_the_last_vnodes(seed, monkeypatch):
     batch, _ = make_batch(prompts, outputs, prefixes, max_ctx=256)
     plain = small_meta(kv_split_sizes=(8, 8), launch_order=False)
     prepare_for_fasttree_meta(batch, plain)
-    monkeypatch.setattr(planner, "FULL_MACHINE_BLOCKS", 1)
+    monkeypatch.setattr(launch_schedule, "MIN_PROGRAM_TILES", 0.0)   # cut every launch anew
     meta = small_meta(kv_split_sizes=(8, 8))
     prepare_for_fasttree_meta(batch, meta)
     assert sum(meta.phase_node_nums) < sum(plain.phase_node_nums), "chunks were joined"
@@ -285,13 +287,14 @@ class FakePool:
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("joined", [False, True])
+@pytest.mark.parametrize("joined", [False, True, "reference_order"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_hook_matches_dense_attention(device, dtype, joined, monkeypatch):
-    """`joined`: 32-token KV splits with the launch order's chunk rule forced on every chain, so
-    that the step after it grows vnodes that were given other vnodes' chunks."""
+    """`joined`: 32-token KV splits with every launch cut anew into block programs, so that the
+    step after it grows tail vnodes that sit at other positions than the planner gave them;
+    "reference_order": FastTreeMetadata(launch_order=False), the reference's own lists."""
     import fasttree_oracle as oracle
-    from fasttree_hip import planner
+    from fasttree_hip import launch_schedule
     from helpers import assert_parity
 
     rng = random.Random(7)
@@ -308,8 +311,10 @@ def test_hook_matches_dense_attention(device, dtype, joined, monkeypatch):
     rows = list(range(n))
     rng.shuffle(rows)
     batch, n_slots = make_batch(prompts, outputs, prefixes, device=device, max_ctx=256, row_of=rows)
-    if joined:
-        monkeypatch.setattr(planner, "FULL_MACHINE_BLOCKS", 1)
+    if joined == "reference_order":
+        meta = small_meta(device=device, launch_order=False)
+    elif joined:
+        monkeypatch.setattr(launch_schedule, "MIN_PROGRAM_TILES", 0.0)
         meta = small_meta(device=device, TSQs=(256 // 4, 16 // 4), kv_split_sizes=(32, 16))
     else:
         meta = small_meta(device=device, TSQs=(256 // 4, 16 // 4))
@@ -431,3 +436,18 @@ def test_hook_with_the_fused_store(device):
     paths = [table[r, : lens[r]].cpu().long() for r in range(n)]
     want = oracle.dense_attention(q.view(n, hq, d).cpu(), k_pool.cpu(), v_pool.cpu(), paths, layer.scaling)
     assert_parity(o.view(n, hq, d).cpu(), want, "hook, fused store", out_dtype=dtype)
+
+
+def test_plan_is_reused_only_for_the_very_same_requests():
+    """The hook re-plans unless the batch holds, one by one, the request objects the plan was
+    made for; the kept tuple owns them, so an address cannot come back under a new request."""
+    from fasttree_hip.sglang_plugin import same_requests
+    a, b, c = Obj(), Obj(), Obj()
+    kept = (a, b)
+    assert same_requests(kept, [a, b]) and same_requests(kept, (a, b))
+    assert not same_requests(None, [a, b]) and not same_requests(kept, [b, a])
+    assert not same_requests(kept, [a]) and not same_requests(kept, [a, b, c]) and not same_requests(kept, [a, c])
+    twin = Obj()
+    twin.__dict__.update(b.__dict__)
+    assert not same_requests(kept, [a, twin]), "equal contents are not the same request"
+    assert same_requests((), [])
