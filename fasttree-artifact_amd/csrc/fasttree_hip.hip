@@ -17,6 +17,7 @@
 
 #include <hip/hip_runtime.h>
 #include <algorithm>
+#include <mutex>
 #include <stdint.h>
 
 #include "../../include/fasttree_hip.h"
@@ -1646,6 +1647,37 @@ int check_common(int d, int g, int dtype) {
 
 }  // namespace
 
+// ---------------------------------------------------------------------------------------
+// Scratch of ft_decode_static: the partial results of one decode call (mid_o, then mid_lse) in
+// a device array of the library, for callers that cannot allocate.  Every device the library
+// runs on holds its own copy until the process ends.  In host code the array's name is a
+// stand-in, not a device address: the address on the current device is asked for once per
+// device and kept, and only that pointer is handed to kernels.
+// ---------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[FT_STATIC_SCRATCH_BYTES];
+
+static int static_scratch_of_current_device(char** out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex guard;
+  static char* address[kMaxDevices] = {};
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return FT_ERR_LAUNCH;
+  }
+  std::lock_guard<std::mutex> lock(guard);
+  if (!address[dev]) {
+    char* ptr = nullptr;
+    if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+      (void)hipGetLastError();
+      return FT_ERR_LAUNCH;
+    }
+    address[dev] = ptr;
+  }
+  *out = address[dev];
+  return FT_OK;
+}
+
 extern "C" {
 
 const char* ft_version(void) { return "fasttree_hip 0.1 (gfx950)"; }
@@ -1660,6 +1692,7 @@ const char* ft_error_string(int code) {
     case FT_ERR_ALIGNMENT: return "pointer or stride not aligned as required";
     case FT_ERR_ARGUMENT: return "argument out of range";
     case FT_ERR_LAUNCH: return "kernel launch failed";
+    case FT_ERR_SCRATCH: return "partial results do not fit the library's static scratch (FT_STATIC_SCRATCH_BYTES)";
     default: return "unknown error";
   }
 }
@@ -1856,6 +1889,35 @@ int ft_decode_programs(const void* q, const void* k, const void* v, void* o,
     return rc;
   return ft_stage2(req_to_vnode_entries, req_to_vnode_offs, req_to_vnode_lens, mid_o, so0, so1, mid_lse, sl0, o, oo0,
                    oo1, batch_size, num_qo_heads, head_dim, dtype, stream);
+}
+
+int ft_decode_static(const void* q, const void* k, const void* v, void* o,
+                     int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+                     int64_t oo0, int64_t oo1,
+                     const int32_t* vnode_to_kv_entries, const int32_t* vnode_to_kv_offs,
+                     const int32_t* vnode_to_kv_lens, const int32_t* vnode_to_q_entries,
+                     const int32_t* vnode_to_q_offs, const int32_t* vnode_to_q_lens,
+                     const int32_t* req_to_vnode_entries, const int32_t* req_to_vnode_offs,
+                     const int32_t* req_to_vnode_lens, int64_t num_rows,
+                     const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
+                     const int32_t* prog_table, int num_programs, int narrow_in_programs,
+                     int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
+                     float sm_scale, int dtype, ft_stream_t stream) {
+  if (num_rows < 0 || num_qo_heads < 1 || head_dim < 1) return FT_ERR_ARGUMENT;
+  // mid_o: num_rows x num_qo_heads x head_dim floats, then (256-byte aligned) mid_lse: num_rows x num_qo_heads
+  const unsigned __int128 o_bytes = (unsigned __int128)num_rows * (unsigned)num_qo_heads * (unsigned)head_dim * 4u;
+  const unsigned __int128 lse_at = (o_bytes + 255u) / 256u * 256u;
+  const unsigned __int128 need = lse_at + (unsigned __int128)num_rows * (unsigned)num_qo_heads * 4u;
+  if (need > (unsigned __int128)FT_STATIC_SCRATCH_BYTES) return FT_ERR_SCRATCH;
+  char* base = nullptr;
+  if (int rc = static_scratch_of_current_device(&base)) return rc;
+  float* mid_o = reinterpret_cast<float*>(base);
+  float* mid_lse = reinterpret_cast<float*>(base + (size_t)lse_at);
+  return ft_decode_programs(q, k, v, o, sq0, sq1, sk0, sk1, sv0, sv1, oo0, oo1, vnode_to_kv_entries, vnode_to_kv_offs,
+                            vnode_to_kv_lens, vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, req_to_vnode_entries,
+                            req_to_vnode_offs, req_to_vnode_lens, mid_o, (int64_t)num_qo_heads * head_dim, head_dim,
+                            mid_lse, num_qo_heads, phase_node_nums, phase_node_offsets, prog_table, num_programs,
+                            narrow_in_programs, batch_size, num_qo_heads, num_kv_heads, head_dim, sm_scale, dtype, stream);
 }
 
 int ft_decode(const void* q, const void* k, const void* v, void* o,

@@ -101,6 +101,44 @@ def fasttree_decode(
     _lib.check(rc, "ft_decode")
 
 
+def fasttree_decode_static(q, k_buffer, v_buffer, o, vnode_to_kv_entries, vnode_to_kv_offs, vnode_to_kv_lens,
+                           vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, req_to_vnode_entries,
+                           req_to_vnode_offs, req_to_vnode_lens, phase_node_nums, phase_node_offsets, sm_scale):
+    """The decode call for callers that cannot allocate device memory (``ft_decode_static``):
+    the partial results go to an array inside the library instead of ``mid_o`` / ``mid_lse``
+    tensors, and neither this wrapper nor the library allocates on the device.  Not in the
+    reference, whose caller allocates both buffers (kernel_bench/fasttree.py:264-269).
+
+    Takes the lists of ``fasttree_preparation(launch_order=True)`` (``phase_node_nums`` carries
+    the program table when there are wide vnodes).  Raises ``FastTreeLibraryError`` when the scratch rows
+    do not fit the library's array (128 MiB per device).  Calls that overlap on one device race
+    on that array."""
+    assert q.shape[-1] == k_buffer.shape[-1]
+    _need_gpu(q, k_buffer, v_buffer, o, vnode_to_kv_entries)
+    _need_inner_contiguous(q, k_buffer, v_buffer, o)
+    _need_i32(vnode_to_kv_entries, vnode_to_kv_offs, vnode_to_kv_lens, vnode_to_q_entries, vnode_to_q_offs,
+              vnode_to_q_lens, req_to_vnode_entries, req_to_vnode_offs, req_to_vnode_lens)
+    if k_buffer.dtype != q.dtype or v_buffer.dtype != q.dtype or o.dtype != q.dtype:
+        raise _lib.FastTreeLibraryError("q, k, v and o must share one dtype")
+    lib = _lib.load()
+    programs = getattr(phase_node_nums, "prog_table", None)
+    rc = lib.ft_decode_static(
+        q.data_ptr(), k_buffer.data_ptr(), v_buffer.data_ptr(), o.data_ptr(),
+        q.stride(0), q.stride(1), k_buffer.stride(0), k_buffer.stride(1),
+        v_buffer.stride(0), v_buffer.stride(1), o.stride(0), o.stride(1),
+        vnode_to_kv_entries.data_ptr(), vnode_to_kv_offs.data_ptr(), vnode_to_kv_lens.data_ptr(),
+        vnode_to_q_entries.data_ptr(), vnode_to_q_offs.data_ptr(), vnode_to_q_lens.data_ptr(),
+        req_to_vnode_entries.data_ptr(), req_to_vnode_offs.data_ptr(), req_to_vnode_lens.data_ptr(),
+        int(vnode_to_q_entries.numel()),
+        _lib.int32_pair(phase_node_nums), _lib.int32_pair(phase_node_offsets),
+        programs.data_ptr() if programs is not None else None,
+        int(getattr(phase_node_nums, "num_programs", 0)), int(getattr(phase_node_nums, "narrow_in_programs", 0)),
+        q.shape[0], q.shape[1], k_buffer.shape[1], q.shape[-1],
+        float(sm_scale), _dtype_code(q), _stream_handle(q),
+    )
+    _lib.check(rc, "ft_decode_static")
+
+
 def fasttree_decode_stage1(q, k_buffer, v_buffer, vnode_to_kv_entries, vnode_to_kv_offs, vnode_to_kv_lens,
                            vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, sm_scale, mid_o, mid_lse,
                            phase_node_nums, phase_node_offsets, phase_q_tile_sizes, phase_kv_tile_sizes):

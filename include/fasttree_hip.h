@@ -43,7 +43,8 @@ enum {
   FT_ERR_GROUP = -4,
   FT_ERR_ALIGNMENT = -5,
   FT_ERR_ARGUMENT = -6,
-  FT_ERR_LAUNCH = -7
+  FT_ERR_LAUNCH = -7,
+  FT_ERR_SCRATCH = -8        /* ft_decode_static: more partial results than FT_STATIC_SCRATCH_BYTES hold */
 };
 
 /* Library version string, e.g. "fasttree_hip 0.1 (gfx950)". */
@@ -156,6 +157,38 @@ int ft_decode_programs(const void* q, const void* k, const void* v, void* o,
                        const int32_t* prog_table, int num_programs, int narrow_in_programs,
                        int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
                        float sm_scale, int dtype, ft_stream_t stream);
+
+/*
+ * ft_decode_programs for callers that cannot allocate device memory (code under HIP graph
+ * capture, serving loops and harnesses that forbid hipMalloc): the partial results live in a
+ * device array of the library instead of mid_o / mid_lse buffers of the caller.  No counterpart
+ * in the reference, whose caller allocates both (kernel_bench/fasttree.py:264-269).  The call
+ * allocates and frees nothing on host-visible APIs: no hipMalloc, no hipFree, no library routine
+ * that allocates.
+ *
+ * num_rows is the number of scratch rows the lists refer to (the length of vnode_to_q_entries).
+ * The array holds FT_STATIC_SCRATCH_BYTES on every device the library is used on, for the life
+ * of the process; a call needs num_rows * num_qo_heads * head_dim * 4 bytes, rounded up to 256,
+ * plus num_rows * num_qo_heads * 4, and returns FT_ERR_SCRATCH when that is more.  The first
+ * call on a device looks up the array's address on that device (make it before a capture
+ * starts); later calls on that device only launch the two kernels.  All calls on one device
+ * share the array: calls that overlap in time on one device (two streams, two threads) race on
+ * it, and its contents are only meaningful between the two launches of one call.  Nothing in it
+ * needs clearing: the first launch writes every row the second one reads.
+ */
+#define FT_STATIC_SCRATCH_BYTES (128u << 20)
+int ft_decode_static(const void* q, const void* k, const void* v, void* o,
+                     int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+                     int64_t oo0, int64_t oo1,
+                     const int32_t* vnode_to_kv_entries, const int32_t* vnode_to_kv_offs,
+                     const int32_t* vnode_to_kv_lens, const int32_t* vnode_to_q_entries,
+                     const int32_t* vnode_to_q_offs, const int32_t* vnode_to_q_lens,
+                     const int32_t* req_to_vnode_entries, const int32_t* req_to_vnode_offs,
+                     const int32_t* req_to_vnode_lens, int64_t num_rows,
+                     const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
+                     const int32_t* prog_table, int num_programs, int narrow_in_programs,
+                     int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
+                     float sm_scale, int dtype, ft_stream_t stream);
 
 /*
  * Decode attention without prefix sharing over a per-request gathered, padded cache
