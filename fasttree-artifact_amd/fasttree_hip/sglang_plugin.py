@@ -53,6 +53,7 @@ class FastTreeMetadata:
         max_batch_size: int = 8192,
         fused_store: bool = False,
         launch_order: bool = True,
+        fix_enumerate: bool = False,
     ):
         self.num_qo_heads = num_qo_heads
         self.num_kv_heads = num_kv_heads
@@ -71,6 +72,11 @@ class FastTreeMetadata:
         #: not in the reference: the vnode lists are arranged as block programs for the kernels
         #: (launch_schedule.block_programs) instead of left in the reference's order
         self.launch_order = launch_order
+        #: not in the reference: evaluate the cost model and merge nodes into their children where
+        #: it says so (what schedule.py:87-118 sets out to do; as shipped its loop over
+        #: ``enumerate(node.children.values())`` never finds a child and nothing is ever merged).
+        #: Off by default = the shipped behaviour.
+        self.fix_enumerate = fix_enumerate
 
         def ints(n):
             return torch.empty(n, dtype=torch.int32, device=device)
@@ -180,18 +186,59 @@ def prepare_for_fasttree_meta(batch, fasttree_metadata: FastTreeMetadata):
     reqs_of = _requests_per_radix_node(batch)
 
     # live nodes in BFS order with the offset of their first token along the path
-    order, token_offset = [], []
-    todo = deque([(root, 0)])
+    order, token_offset, parent_of = [], [], []
+    todo = deque([(root, 0, -1)])
     while todo:
-        node, off = todo.popleft()
+        node, off, up = todo.popleft()
         order.append(node)
         token_offset.append(off)
+        parent_of.append(up)
         for child in node.children.values():
             if child in reqs_of:
-                todo.append((child, off + len(node.value)))
+                todo.append((child, off + len(node.value), len(order) - 1))
 
     n_reqs = [len(reqs_of[node]) if node in reqs_of else 0 for node in order]
     seqlens = [len(node.value) for node in order]
+    merge = bool(getattr(meta, "fix_enumerate", False))
+    own_lens, all_reqs = list(seqlens), [list(reqs_of[node]) if node in reqs_of else [] for node in order]
+    members_of, start_of = None, list(token_offset)
+
+    def decide(q_tiles, kv_tiles):
+        """The cost model's decisions for the current tile sizes: per node the requests its own
+        vnodes serve, the tokens they attend (its own and those of the ancestors merged into
+        it) and where that run starts along the path."""
+        from .kv_tree import KVTreeNode
+        from .planner import FastTreeParams, _run_chain, _tree_heuristic
+
+        params = FastTreeParams()
+        params.set_values(meta.alpha, meta.beta, meta.gamma)
+        params.set_q_tile_sizes(list(q_tiles)); params.set_kv_tile_sizes(list(kv_tiles))
+        params.set_kv_group_num(meta.kv_group_num)
+        info = []
+        for i, up in enumerate(parent_of):
+            n = KVTreeNode(parent=up, id=i, seqlen=own_lens[i])
+            n.requests = all_reqs[i] if i else list(range(len(batch.reqs)))
+            info.append(n)
+        for up in parent_of[1:]:
+            info[up].num_children += 1
+        assignment = _tree_heuristic(info, params)
+        children = [[] for _ in order]
+        for c, up in enumerate(parent_of):
+            if up >= 0:
+                children[up].append(c)
+        served = []
+        for i in range(len(order)):
+            gone = set(r for c in children[i] if assignment[c] == 1 for r in all_reqs[c])
+            listed = [r for c in children[i] if assignment[c] == 0 for r in all_reqs[c]]  # child by child, as the reference lists them
+            seen = set(listed) | gone
+            listed += [r for r in all_reqs[i] if r not in seen]             # requests whose prompt ends at this node
+            served.append(listed if i else [])
+        lens, starts = [], []
+        for i in range(len(order)):
+            chain, total = _run_chain(info, assignment, i) if i else ([0], 0)
+            lens.append(total)
+            starts.append(token_offset[chain[0]])
+        return served, lens, starts
 
     q_tiles = meta.TSQs
     kv_tiles = meta.TSKs
@@ -206,6 +253,9 @@ def prepare_for_fasttree_meta(batch, fasttree_metadata: FastTreeMetadata):
         return [x * meta.num_kv_heads for x in p]
 
     for it in range(3):
+        if merge:
+            members_of, seqlens, start_of = decide(q_tiles, kv_tiles)
+            n_reqs = [len(m) for m in members_of]
         p = parallelism()
         if it == 0:
             low = [ph for ph in range(2) if 0 < p[ph] < meta.para_threshs1[ph]]
@@ -240,14 +290,20 @@ def prepare_for_fasttree_meta(batch, fasttree_metadata: FastTreeMetadata):
                 q_offs.append(q0 + s)
                 q_lens.append(min(s + q_tile, n_q) - s)
 
-    for node, nq, length, off in zip(order, n_reqs, seqlens, token_offset):
+    if merge:
+        members_of, seqlens, start_of = decide(q_tiles, kv_tiles)   # (for the tile sizes the passes settled on)
+        n_reqs = [len(m) for m in members_of]
+    for i, (node, nq, length, off) in enumerate(zip(order, n_reqs, seqlens, start_of)):
         if nq == 0:
             continue
         # the members are listed child by child where the node has live children (all of them
         # keep assignment 0), else from the node itself; the KV is read through the row of the
         # first member
-        groups = [c for c in node.children.values() if c in reqs_of] or [node]
-        members = [r for grp in groups for r in reqs_of[grp]]
+        if merge:
+            members = members_of[i]
+        else:
+            groups = [c for c in node.children.values() if c in reqs_of] or [node]
+            members = [r for grp in groups for r in reqs_of[grp]]
         phase = 0 if nq > q_tiles[1] else 1
         emit(stride * int(rows[members[0]]) + off, length, members, q_tiles[phase], kv_splits[phase], nq)
 

@@ -84,19 +84,24 @@ CONFIGS = {
     "c2": ([1, 64], [4096, 256], 32, 8, torch.float16, 2),
     "c3": ([1, 10, 400], [4000, 400, 40], 32, 8, torch.float16, 3),
 }
-# (q tiles, kv split sizes, thresholds 1, thresholds 2): the reference bench's values and a
-# preset sized for 256 compute units with 64-request tiles
+# (q tiles, kv split sizes, thresholds 1, thresholds 2): the reference bench's values
+# (kernel_bench/benchmark.py:246-254), the preset bench.py measures (thresholds for 256 compute
+# units, 256-token splits for phases short of parallelism), and 64-request tiles
 PRESETS = {
     "reference_defaults": (None, (1024, 128), (132, 528), (132, 132)),
+    "mi355x": (None, (1024, 256), (256, 1024), (256, 256)),
     "wide_tiles": ("wide", (1024, 128), (256, 1024), (256, 256)),
 }
+ORDERS = {"planner_order": False, "launch_order": True}
 
 
+@pytest.mark.parametrize("order", list(ORDERS))
 @pytest.mark.parametrize("preset", list(PRESETS))
 @pytest.mark.parametrize("name", list(CONFIGS))
-def test_baseline_configs_against_dense_oracle(name, preset, device):
-    """C1-C3 at full size, shuffled paged pool: every request against the fp64 oracle."""
-    _announce(name, preset)
+def test_baseline_configs_against_dense_oracle(name, preset, order, device):
+    """C1-C3 at full size, shuffled paged pool: every request against the fp64 oracle, with the
+    reference's lists and with the lists arranged as block programs."""
+    _announce(name, preset, order)
     sizes, lens, hq, hkv, dtype, seed = CONFIGS[name]
     tree, ptrs, batch = build_tree({"kind": "regular", "sizes": sizes, "lens": lens})
     inp = make_decode_inputs(tree, hq, hkv, 128, device=device, dtype=dtype, seed=seed, shuffle_slots=True)
@@ -107,10 +112,11 @@ def test_baseline_configs_against_dense_oracle(name, preset, device):
     params.set_values(0.66, 0.33, 0.1); params.set_q_tile_sizes(list(q_tiles)); params.set_kv_tile_sizes([32, 32])
     params.set_kv_group_num(g)
     aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, hq, hkv, 128, list(splits), list(thr1), list(thr2), params,
-                                  device=device, kv_slot_map=inp.slot_map)
+                                  device=device, kv_slot_map=inp.slot_map, launch_order=ORDERS[order])
+    assert (type(aux[11]) is list) != ORDERS[order]
     o = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, q_tiles, [32, 32], 1.0 / math.sqrt(128))
     sample = None if batch <= 64 else list(range(0, batch, 7))
-    print(_dense_check(tree, inp, o, f"{name}/{preset}", sample), flush=True)
+    print(_dense_check(tree, inp, o, f"{name}/{preset}/{order}", sample), flush=True)
     # every request against an fp32 torch attention on the device (gathered per request)
     k_cache, v_cache, lens_t = gather_per_request(inp)
     mask = torch.arange(k_cache.shape[1], device=device)[None, :] < lens_t[:, None]
@@ -151,25 +157,27 @@ def test_launch_order_does_not_change_the_result(spec, device):
         print(_dense_check(tree, inp, o, "launch order", list(range(0, batch, 5 if batch < 600 else 37))), flush=True)
 
 
+@pytest.mark.parametrize("order", list(ORDERS))
 @pytest.mark.parametrize("seed", [0, 1, 2])
-def test_deep_irregular_tree(seed, device):
+def test_deep_irregular_tree(seed, order, device):
     """C5: 5 levels, fan-out U[1,8], lengths log-uniform [16,2048], <= 1024 leaves, GQA 8."""
-    _announce("c5", seed)
+    _announce("c5", seed, order)
     tree, ptrs, batch = build_tree({"kind": "irregular", "seed": seed})
     inp = make_decode_inputs(tree, 64, 8, 128, device=device, dtype=torch.float16, seed=seed, shuffle_slots=True)
     params = FastTreeParams()
     params.set_q_tile_sizes([8, 2]); params.set_kv_tile_sizes([32, 32]); params.set_kv_group_num(8)
     aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, 64, 8, 128, [1024, 128], [132, 528], [132, 132], params,
-                                  device=device, kv_slot_map=inp.slot_map)
+                                  device=device, kv_slot_map=inp.slot_map, launch_order=ORDERS[order])
     o = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, list(params.TSQs), [32, 32], 1.0 / math.sqrt(128))
     step = max(1, batch // 48)
     print(_dense_check(tree, inp, o, f"c5 seed {seed}", list(range(0, batch, step))), flush=True)
 
 
-def test_wide_shallow_tree_bf16(device):
+@pytest.mark.parametrize("order", list(ORDERS))
+def test_wide_shallow_tree_bf16(order, device):
     """C4: 512-token root, 2048 leaves of 1024 tokens, bf16, > 2^31 pool elements (needs
     64-bit addressing).  Sampled requests against the fp64 oracle."""
-    _announce("c4")
+    _announce("c4", order)
     tree, ptrs, batch = build_tree({"kind": "regular", "sizes": [1, 2048], "lens": [512, 1024]})
     inp = make_decode_inputs(tree, 32, 8, 128, device=device, dtype=torch.bfloat16, seed=4, shuffle_slots=True,
                              host_rng=False)
@@ -177,7 +185,7 @@ def test_wide_shallow_tree_bf16(device):
     params = FastTreeParams()
     params.set_q_tile_sizes([16, 4]); params.set_kv_tile_sizes([32, 32]); params.set_kv_group_num(4)
     aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, 32, 8, 128, [1024, 128], [132, 528], [132, 132], params,
-                                  device=device, kv_slot_map=inp.slot_map)
+                                  device=device, kv_slot_map=inp.slot_map, launch_order=ORDERS[order])
     o = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, [16, 4], [32, 32], 1.0 / math.sqrt(128))
     high = [r for r in range(batch) if int(inp.path_tokens[r].max()) * 8 * 128 >= 2 ** 31]
     assert high, "some request must read pool rows beyond 2^31 elements"
@@ -197,8 +205,9 @@ def test_wide_shallow_tree_bf16(device):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
 @pytest.mark.parametrize("d", [32, 64, 128, 256])
 @pytest.mark.parametrize("heads", [(4, 4), (8, 2), (16, 2), (16, 1)], ids=["mha", "gqa4", "gqa8", "gqa16"])
-def test_head_dims_groups_and_dtypes(heads, d, dtype, device):
-    _announce("shape sweep", heads, d, dtype)
+@pytest.mark.parametrize("order", list(ORDERS))
+def test_head_dims_groups_and_dtypes(order, heads, d, dtype, device):
+    _announce("shape sweep", order, heads, d, dtype)
     hq, hkv = heads
     g = hq // hkv
     tree, ptrs, batch = build_tree({"kind": "irregular", "seed": 21, "levels": 4, "fanout_range": (1, 5),
@@ -208,9 +217,9 @@ def test_head_dims_groups_and_dtypes(heads, d, dtype, device):
     params = FastTreeParams()
     params.set_q_tile_sizes(list(q_tiles)); params.set_kv_tile_sizes([32, 32]); params.set_kv_group_num(g)
     aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, hq, hkv, d, [256, 64], [132, 528], [132, 132], params,
-                                  device=device, kv_slot_map=inp.slot_map)
+                                  device=device, kv_slot_map=inp.slot_map, launch_order=ORDERS[order])
     o = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, list(params.TSQs), list(params.TSKs), 1.0 / math.sqrt(d))
-    _dense_check(tree, inp, o, f"{heads} d={d} {dtype}", dtype=dtype)
+    _dense_check(tree, inp, o, f"{order} {heads} d={d} {dtype}", dtype=dtype)
 
 
 def test_stage_outputs_against_restated_arithmetic(device):

@@ -287,12 +287,13 @@ class FakePool:
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("joined", [False, True, "reference_order"])
+@pytest.mark.parametrize("joined", [False, True, "reference_order", "merged", "merged_reference_order"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_hook_matches_dense_attention(device, dtype, joined, monkeypatch):
     """`joined`: 32-token KV splits with every launch cut anew into block programs, so that the
     step after it grows tail vnodes that sit at other positions than the planner gave them;
-    "reference_order": FastTreeMetadata(launch_order=False), the reference's own lists."""
+    "reference_order": FastTreeMetadata(launch_order=False), the reference's own lists;
+    "merged...": FastTreeMetadata(fix_enumerate=True) with nodes merged into their children."""
     import fasttree_oracle as oracle
     from fasttree_hip import launch_schedule
     from helpers import assert_parity
@@ -313,6 +314,10 @@ def test_hook_matches_dense_attention(device, dtype, joined, monkeypatch):
     batch, n_slots = make_batch(prompts, outputs, prefixes, device=device, max_ctx=256, row_of=rows)
     if joined == "reference_order":
         meta = small_meta(device=device, launch_order=False)
+    elif joined in ("merged", "merged_reference_order"):
+        # the cost model evaluated (fix_enumerate) with a reduction cost that merges every shared node
+        meta = small_meta(device=device, fix_enumerate=True, gamma=50.0, para_threshs1=(0, 0), para_threshs2=(0, 0),
+                          launch_order=joined == "merged")
     elif joined:
         monkeypatch.setattr(launch_schedule, "MIN_PROGRAM_TILES", 0.0)
         meta = small_meta(device=device, TSQs=(256 // 4, 16 // 4), kv_split_sizes=(32, 16))
@@ -451,3 +456,63 @@ def test_plan_is_reused_only_for_the_very_same_requests():
     twin.__dict__.update(b.__dict__)
     assert not same_requests(kept, [a, twin]), "equal contents are not the same request"
     assert same_requests((), [])
+
+
+@pytest.mark.parametrize("launch_order", [False, True])
+@pytest.mark.parametrize("gamma", [0.1, 50.0])
+@pytest.mark.parametrize("seed", range(6))
+def test_merge_path_keeps_what_every_request_attends(seed, gamma, launch_order):
+    """FastTreeMetadata(fix_enumerate=True): the cost model is evaluated and nodes are merged
+    into their children (with a large gamma: wherever the model is asked).  Whatever it decides,
+    every request attends each of its tokens exactly once through the rows listed for it --
+    also requests whose prompt ends at an inner node of the radix tree -- and its last vnode is
+    still the single-request vnode that ends where its tokens end."""
+    rng = random.Random(500 + seed)
+    system = [rng.randint(1, 10**6) for _ in range(rng.randint(5, 90))]
+    prefixes, prompts, outputs = [system], [], []
+    for _ in range(rng.randint(1, 4)):
+        mid = system + [rng.randint(1, 10**6) for _ in range(rng.randint(1, 60))]
+        prefixes.append(mid)
+        if rng.random() < 0.5:
+            prompts.append(list(mid)); outputs.append([rng.randint(1, 10**6) for _ in range(rng.randint(0, 9))])   # ends at an inner node
+        for _ in range(rng.randint(1, 12)):
+            prompts.append(mid + [rng.randint(1, 10**6) for _ in range(rng.randint(1, 40))])
+            outputs.append([rng.randint(1, 10**6) for _ in range(rng.randint(0, 12))])
+    batch, _ = make_batch(prompts, outputs, prefixes, max_ctx=256)
+    meta = small_meta(kv_split_sizes=(16, 8), gamma=gamma, fix_enumerate=True, launch_order=launch_order)
+    prepare_for_fasttree_meta(batch, meta)
+    table = batch.req_to_token_pool.req_to_token
+    got = plan_lists(meta, batch)
+    for r, slots in enumerate(covered_slots(meta, batch)):
+        assert sorted(slots) == sorted(table[r, : len(prompts[r]) + len(outputs[r]) + 1].tolist()), r
+        rows = got["req_entries"][got["req_offs"][r]: got["req_offs"][r] + got["req_lens"][r]]
+        assert rows == sorted(set(rows)) and all(got["q_entries"][i] == r for i in rows)
+        v = meta.req_last_vnodes[r]
+        assert got["q_lens"][v] == 1 and got["q_entries"][got["q_offs"][v]] == r
+        assert got["kv_offs"][v] + got["kv_lens"][v] == r * table.stride(0) + len(prompts[r]) + len(outputs[r]) + 1
+    assert sum(got["req_lens"]) == len(got["q_entries"])
+
+
+def test_merge_path_hand_derived():
+    """A=[1,2,3,4] -> B=[5,6] (request 0), C=[7,8,9] (requests 1, 2).  With a reduction cost of
+    50 per query the model merges A into both children: request 0 attends A+B as one run of 6
+    tokens through its own row, requests 1 and 2 attend A+C as one run of 7 through the row of
+    request 1; A keeps no vnode.  With the default cost (0.1) nothing is merged and the plan is
+    the shipped one."""
+    prompts = [[1, 2, 3, 4, 5, 6], [1, 2, 3, 4, 7, 8, 9], [1, 2, 3, 4, 7, 8, 9]]
+    outputs = [[10, 11], [12], []]
+    batch, _ = make_batch(prompts, outputs, shared_prefixes=[[1, 2, 3, 4]], row_of=[2, 0, 5])
+    s = 64
+    # (thresholds of 0: the tile sizes stay as given; with the default thresholds this small batch
+    # ends up with 16-request tiles, for which the model does not merge)
+    meta = small_meta(launch_order=False, fix_enumerate=True, gamma=50.0, para_threshs1=(0, 0), para_threshs2=(0, 0))
+    prepare_for_fasttree_meta(batch, meta)
+    got = plan_lists(meta, batch)
+    assert got["kv_offs"] == [2 * s + 0, 0 * s + 0, 2 * s + 6, 0 * s + 7, 5 * s + 7]
+    assert got["kv_lens"] == [6, 7, 3, 2, 1]
+    assert got["q_lens"] == [1, 2, 1, 1, 1] and got["q_entries"] == [0, 1, 2, 0, 1, 2]
+    assert got["req_lens"] == [2, 2, 2] and meta.req_last_vnodes == [2, 3, 4]
+    shipped, same = small_meta(launch_order=False), small_meta(launch_order=False, fix_enumerate=True)
+    prepare_for_fasttree_meta(batch, shipped)
+    prepare_for_fasttree_meta(batch, same)
+    assert plan_lists(same, batch) == plan_lists(shipped, batch)
