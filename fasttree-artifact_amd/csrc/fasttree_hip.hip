@@ -849,9 +849,12 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, cons
         __syncthreads();
       }
     };
-    // rows of super tile j -> ring buffer j % kBufs.  Tokens past the run repeat its last token: the
-    // scores of such rows are masked and their V rows are finite.
-    auto issue_rows = [&](int j) {
+    // rows of super tile j -> ring buffer j % kBufs, in two steps: read_rows(j) takes the slot
+    // indices of the rows this wave loads out of LDS (one super tile ahead of the loads, so that
+    // the LDS round trip is hidden by a tile step), issue_rows(j) requests the rows.  Tokens past
+    // the run repeat its last token: the scores of such rows are masked and their V rows are finite.
+    unsigned srow[W::kSlots];
+    auto read_rows = [&](int j) {
       if (j >= nsuper) return;
       if constexpr (!GATHERED) {
         if (j * W::kTokens >= idx_base + W::kIdxCap) {  // block uniform
@@ -859,30 +862,35 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, cons
           stage_indices(idx_base + W::kIdxCap);
         }
       }
-      const unsigned buf = ring + (unsigned)(j % W::kBufs) * W::kBytes;
-      unsigned srow[W::kSlots];
-      unsigned chunk[W::kSlots];
 #pragma unroll
       for (int u = 0; u < W::kSlots; ++u) {
         const int grp = W::kGroups >= kWideWaves ? u * kWideWaves + wave : wave % W::kGroups;
         const int row = grp * W::kGroupRows + grp_row;
         const int t = min(j * W::kTokens + row, vn.kv_len - 1);
         srow[u] = GATHERED ? (unsigned)(vn.kv_base + t) : (unsigned)idx_lds[t - idx_base];
-        chunk[u] = 16 * (pos ^ W::swz(row));
       }
+    };
+    auto issue_rows = [&](int j) {
+      if (j >= nsuper) return;
+      const unsigned buf = ring + (unsigned)(j % W::kBufs) * W::kBytes;
 #pragma unroll
       for (int u = 0; u < W::kUnits; ++u) {
         // unit u of this wave: K groups first, then V groups
         const bool is_v = W::kGroups >= kWideWaves ? u >= W::kSlots : wave >= W::kGroups;
         const int sl = u % W::kSlots;
         const int grp = W::kGroups >= kWideWaves ? sl * kWideWaves + wave : wave % W::kGroups;
+        const int row = grp * W::kGroupRows + grp_row;
         const char* src = (is_v ? vbase : kbase) + (uint64_t)srow[sl] * (is_v ? v_stride : k_stride);
-        load_direct16(src + chunk[sl], buf + (is_v ? W::kBytesK : 0) + grp * 1024);
+        load_direct16(src + 16 * (pos ^ W::swz(row)), buf + (is_v ? W::kBytesK : 0) + grp * 1024);
       }
     };
     if (nsuper > 0) stage_indices(0);  // block uniform
 #pragma unroll
-    for (int j = 0; j < W::kAhead; ++j) issue_rows(j);
+    for (int j = 0; j < W::kAhead; ++j) {
+      read_rows(j);
+      issue_rows(j);
+    }
+    read_rows(W::kAhead);
     load_q_frags32<D>(q_src, qf);
     // nothing the compiler itself tracks (the Q fragments) may still be in flight in the loop:
     // a wait for it there would also wait for every direct load
@@ -899,6 +907,7 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, cons
       __syncthreads();
       // the buffer consumed before that barrier is free: refill it
       issue_rows(super + W::kAhead);
+      read_rows(super + W::kAhead + 1);
       if (active) {
         const WideLane la = at_buffer(la0, cur);
 #pragma unroll 1
