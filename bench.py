@@ -143,6 +143,9 @@ def main():
     ap.add_argument("--kv-splits", default=None, help="override the preset's KV split sizes, e.g. 1024,128")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gathered", action="store_true")
+    ap.add_argument("--phase", default="both", choices=["both", "wide", "narrow"],
+                    help="with --profile-only: launch only the first stage, restricted to the block programs "
+                         "(wide) or to the vnodes served one wave each (narrow), for per-phase kernel traces")
     ap.add_argument("--profile-only", action="store_true",
                     help="run warm-up + steps back to back and exit (for rocprofv3)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -187,6 +190,19 @@ def main():
         fasttree_decode(inp.Q, inp.K_pool, inp.V_pool, o, *aux, prob["q_tiles"], prob["kv_tiles"], scale)
 
     nums, offs = aux[11], aux[12]  # (the phase list carries the program table: passed as it is)
+    if args.phase != "both":
+        if not args.profile_only:
+            log("bench.py: --phase is for --profile-only runs")
+            sys.exit(2)
+        from fasttree_hip.launch_schedule import LaunchPhases
+        part = LaunchPhases([nums[0], 0] if args.phase == "wide" else [0, nums[1]])
+        if args.phase == "wide":
+            part.prog_table = getattr(nums, "prog_table", None)
+            part.num_programs = getattr(nums, "num_programs", 0)
+        elif getattr(nums, "narrow_in_programs", 0):
+            log("bench.py: the narrow vnodes of this plan are served inside the block programs")
+            sys.exit(2)
+        nums = part
 
     def stage1():
         fasttree_decode_stage1(inp.Q, inp.K_pool, inp.V_pool, *aux[:6], scale, aux[9], aux[10], nums, offs,
@@ -199,6 +215,12 @@ def main():
     # for the wall clock, once more as its two launches (what ft_decode enqueues) with an event on
     # the launch stream before, between and after, for the per-kernel durations -- the events
     # themselves cost a few microseconds per step, which must not leak into ms_per_step.
+    if args.phase != "both":
+        for _ in range(args.warmup + args.steps):
+            stage1()
+        torch.cuda.synchronize()
+        log(f"profile-only: {args.warmup + args.steps} stage-1 launches of the {args.phase} phase, vnodes {list(nums)}")
+        return
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

@@ -1,0 +1,37 @@
+"""bench.py's reported figures are tied to the tracked profile summaries (CPU only)."""
+
+import os
+import re
+import subprocess
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+
+
+def test_measured_traffic_is_read_from_the_tracked_profiles():
+    """`roofline.traffic` of the bench line is the number a profile summary records for that
+    workload, preset and kernel -- for the headline workload there must be one, and it must be the
+    sum of the scaled FETCH_SIZE and WRITE_SIZE figures of the same file."""
+    import bench
+    got = bench.measured_traffic("c3", "mi355x", "stage1", "fp16")
+    assert got is not None and 1e8 < got < 3e8
+    text = open(os.path.join(ROOT, "profiles", "stage1_c3_fp16.txt")).read()
+    m = re.search(r"stage1_fused_kernel<F16, 128, false>\(Stage1Args\)\s+read\s+(\d+) KiB.*?write\s+(\d+) KiB", text)
+    assert m and abs((int(m.group(1)) + int(m.group(2))) * 1024 - got) <= 2048
+    for wl, dt in (("c1", "fp16"), ("c2", "fp16"), ("c4", "bf16"), ("c5", "fp16")):
+        assert bench.measured_traffic(wl, "mi355x", "stage1", dt) is not None, wl
+    assert bench.measured_traffic("c3", "reference", "stage1", "fp16") is None    # no such run is on record
+    assert bench.measured_traffic("c9", "mi355x", "stage1", "fp16") is None
+
+
+def test_profiles_name_the_command_that_made_them():
+    for name in os.listdir(os.path.join(ROOT, "profiles")):
+        text = open(os.path.join(ROOT, "profiles", name)).read()
+        assert "rocprofv3" in text and "bench.py" in text, name
+        assert "_work" not in text and "gpurun" not in text, name
+
+
+def test_more_than_one_gpu_is_refused():
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert out.returncode == 2 and "ONE GPU" in out.stderr
