@@ -140,6 +140,8 @@ struct Stage1Args {
   const int32_t* prog_table;
   int num_programs;
   int narrow_in_programs;          // narrow vnodes (from narrow_begin) that programs serve
+  int real_dim;                    // head dimension of the tensors; smaller than the kernel's D only for head_dim 16,
+                                   // which the per-wave staging kernels compute as a zero-padded 32-dim contraction
   int g;
   int hkv;
   float scale_log2;  // sm_scale * log2(e)
@@ -223,7 +225,7 @@ __device__ __forceinline__ void load_q_frags(const Stage1Args& a, const VnodeVie
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       u32x4 z = {0u, 0u, 0u, 0u};
-      qf[qb][ks] = ok ? *reinterpret_cast<const u32x4*>(src + 64 * ks) : z;
+      qf[qb][ks] = ok && 32 * ks + 8 * c < a.real_dim ? *reinterpret_cast<const u32x4*>(src + 64 * ks) : z;
     }
   }
 }
@@ -367,7 +369,7 @@ __device__ __forceinline__ void wave_attend(const Stage1Args& a, const VnodeView
       u32x4 z = {0u, 0u, 0u, 0u};
       kreg[i] = z;
       vreg[i] = z;
-      if (slot[i] >= 0) {
+      if (slot[i] >= 0 && 8 * ld_chunk < a.real_dim) {   // (chunks past a 16-dim row stay zero)
         const int64_t srow = GATHERED ? (vn.kv_base + slot[i]) : (int64_t)slot[i];
         kreg[i] = *reinterpret_cast<const u32x4*>(kbase + 2 * srow * a.sk0);
         vreg[i] = *reinterpret_cast<const u32x4*>(vbase + 2 * srow * a.sv0);
@@ -418,7 +420,8 @@ __device__ __forceinline__ void write_partials(const Stage1Args& a, const VnodeV
     const float inv = l > 0.f ? 1.f / l : 0.f;
     float* dst = a.mid_o + row * a.so0 + (int64_t)head * a.so1 + 4 * c;
 #pragma unroll
-    for (int db = 0; db < DB; ++db) *reinterpret_cast<f32x4*>(dst + 16 * db) = st.o[qb][db] * inv;
+    for (int db = 0; db < DB; ++db)
+      if (16 * db < a.real_dim) *reinterpret_cast<f32x4*>(dst + 16 * db) = st.o[qb][db] * inv;
     if (c == 0) a.mid_lse[row * a.sl0 + head] = l > 0.f ? (__builtin_amdgcn_logf(l) + st.m[qb]) * kLn2 : -INFINITY;
   }
 }
@@ -1589,9 +1592,9 @@ int launch_stage1_narrow(const Stage1Args& a0, hipStream_t stream) {
 
 // `a` names two vnode ranges: [vnode_begin, +vnode_count) of wide vnodes (more than 16 query
 // rows) and [narrow_begin, +narrow_count) of narrow ones.
-template <typename E, int D, bool GATHERED>
+template <typename E, int D, bool GATHERED, bool STAGED = (D > 128)>
 int launch_stage1_d(const Stage1Args& a, hipStream_t stream) {
-  if constexpr (D > 128) {
+  if constexpr (STAGED) {
     // 128-token double buffers of 512-byte rows do not fit in LDS: per-wave staging kernels
     if (a.vnode_count > 0)
       if (int rc = launch_stage1_inst<E, D, 2, true, GATHERED>(a, a.hkv, stream)) return rc;
@@ -1612,6 +1615,7 @@ template <bool GATHERED>
 int launch_stage1(const Stage1Args& a, int d, int dtype, hipStream_t stream) {
 #define FT_DISPATCH_D(E)                                              \
   switch (d) {                                                        \
+    case 16: return launch_stage1_d<E, 32, GATHERED, true>(a, stream);\
     case 32: return launch_stage1_d<E, 32, GATHERED>(a, stream);      \
     case 64: return launch_stage1_d<E, 64, GATHERED>(a, stream);      \
     case 128: return launch_stage1_d<E, 128, GATHERED>(a, stream);    \
@@ -1635,6 +1639,7 @@ int launch_stage2_inst(const Stage2Args& a, hipStream_t stream) {
 int launch_stage2(const Stage2Args& a, int d, int dtype, hipStream_t stream) {
 #define FT_DISPATCH_D(E)                                       \
   switch (d) {                                                 \
+    case 16: return launch_stage2_inst<E, 16>(a, stream);      \
     case 32: return launch_stage2_inst<E, 32>(a, stream);      \
     case 64: return launch_stage2_inst<E, 64>(a, stream);      \
     case 128: return launch_stage2_inst<E, 128>(a, stream);    \
@@ -1649,7 +1654,7 @@ int launch_stage2(const Stage2Args& a, int d, int dtype, hipStream_t stream) {
 
 int check_common(int d, int g, int dtype) {
   if (dtype != FT_DTYPE_F16 && dtype != FT_DTYPE_BF16) return FT_ERR_DTYPE;
-  if (d != 32 && d != 64 && d != 128 && d != 256) return FT_ERR_HEAD_DIM;
+  if (d != 16 && d != 32 && d != 64 && d != 128 && d != 256) return FT_ERR_HEAD_DIM;
   if (g < 1 || g > 64) return FT_ERR_GROUP;
   return FT_OK;
 }
@@ -1696,7 +1701,7 @@ const char* ft_error_string(int code) {
     case FT_OK: return "ok";
     case FT_ERR_NULL_POINTER: return "null pointer argument";
     case FT_ERR_DTYPE: return "unsupported dtype (fp16 and bf16 only)";
-    case FT_ERR_HEAD_DIM: return "unsupported head dimension (32, 64, 128, 256)";
+    case FT_ERR_HEAD_DIM: return "unsupported head dimension (16, 32, 64, 128, 256)";
     case FT_ERR_GROUP: return "unsupported query/KV head ratio";
     case FT_ERR_ALIGNMENT: return "pointer or stride not aligned as required";
     case FT_ERR_ARGUMENT: return "argument out of range";
@@ -1734,6 +1739,7 @@ static int stage1_setup(Stage1Args& a, const void* q, const void* k, const void*
   a.q_entries = vnode_to_q_entries; a.q_offs = vnode_to_q_offs; a.q_lens = vnode_to_q_lens;
   a.g = kv_group_num;
   a.hkv = num_kv_heads;
+  a.real_dim = head_dim;
   a.scale_log2 = sm_scale * kLog2e;
   a.mid_o = mid_o; a.so0 = so0; a.so1 = so1; a.mid_lse = mid_lse; a.sl0 = sl0;
   return FT_OK;
@@ -1858,7 +1864,7 @@ int ft_stage1_programs(const void* q, const void* k, const void* v,
   if (num_kv_heads < 1 || num_qo_heads % num_kv_heads != 0) return FT_ERR_GROUP;
   const int g = num_qo_heads / num_kv_heads;
   if (int rc = check_common(head_dim, g, dtype)) return rc;
-  if (head_dim > 128) return FT_ERR_HEAD_DIM;  // the program table is for the direct-load kernels
+  if (head_dim < 32 || head_dim > 128) return FT_ERR_HEAD_DIM;  // the program table is for the direct-load kernels
   if (phase_node_nums[0] == 0 && phase_node_nums[1] == 0) return FT_OK;
   Stage1Args a;
   if (int rc = stage1_setup(a, q, k, v, sq0, sq1, sk0, sk1, sv0, sv1, vnode_to_kv_entries, vnode_to_kv_offs,
@@ -1979,6 +1985,7 @@ int ft_gathered_decode(const void* q, const void* k_cache, const void* v_cache,
   else { a.vnode_begin = 0; a.vnode_count = batch_size * nsplit; a.wide_rows = g; }
   a.g = g;
   a.hkv = num_kv_heads;
+  a.real_dim = head_dim;
   a.scale_log2 = sm_scale * kLog2e;
   a.mid_o = mid_o; a.so0 = (int64_t)num_qo_heads * head_dim; a.so1 = head_dim;
   a.mid_lse = mid_lse; a.sl0 = num_qo_heads;

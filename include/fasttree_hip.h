@@ -20,7 +20,8 @@
  *     be multiples of 4, the head stride of mid_lse is 1.
  *   - index arrays are contiguous int32 in device memory.  No element past the ranges
  *     named by the offset/length arrays is ever read.
- *   - D in {32, 64, 128, 256}; Hq = Hkv * g with 1 <= g <= 64; sm_scale > 0.
+ *   - D in {16, 32, 64, 128, 256} (the reference's set, kernel_bench/fasttree.py:439; 16 is computed as a
+ *     zero-padded 32-dim contraction); Hq = Hkv * g with 1 <= g <= 64; sm_scale > 0.
  */
 #ifndef FASTTREE_HIP_H_
 #define FASTTREE_HIP_H_

@@ -203,7 +203,7 @@ def test_wide_shallow_tree_bf16(order, device):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
-@pytest.mark.parametrize("d", [32, 64, 128, 256])
+@pytest.mark.parametrize("d", [16, 32, 64, 128, 256])
 @pytest.mark.parametrize("heads", [(4, 4), (8, 2), (16, 2), (16, 1)], ids=["mha", "gqa4", "gqa8", "gqa16"])
 @pytest.mark.parametrize("order", list(ORDERS))
 def test_head_dims_groups_and_dtypes(order, heads, d, dtype, device):
