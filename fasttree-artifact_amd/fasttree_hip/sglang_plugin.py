@@ -423,6 +423,26 @@ def same_requests(planned_for, reqs) -> bool:
             and all(a is b for a, b in zip(planned_for, reqs)))
 
 
+def plan_or_step(server, batch, replan_every, plan=None, step=None):
+    """What the patched ``forward_decode_batch`` does before every decode forward: a new plan when
+    the batch does not hold the very requests the last plan was made for, or when that plan has
+    served ``replan_every`` forwards; the in-place ``+1`` step otherwise.  The reference plans at
+    the top of every ``forward_step`` and steps between the ``num_continue_decode_steps``
+    forwards of that step (plugin.py:108-131); ``replan_every`` is that number.  ``server`` keeps
+    ``_fasttree_planned_for`` (a tuple of the request objects) and ``_fasttree_forwards``."""
+    plan = plan or prepare_for_fasttree_meta
+    step = step or prepare_for_fasttree_step
+    served = getattr(server, "_fasttree_forwards", 0)
+    if same_requests(getattr(server, "_fasttree_planned_for", None), batch.reqs) and served < replan_every:
+        step(batch, server.fasttree_metadata)
+        server._fasttree_forwards = served + 1
+        return "step"
+    plan(batch, server.fasttree_metadata)
+    server._fasttree_planned_for = tuple(batch.reqs)
+    server._fasttree_forwards = 1
+    return "plan"
+
+
 def load_fasttree_plugin(enable_fasttree=True, annotate_breakdown=False):
     """Installs the hook into SGLang v0.2.13 (plugin.py:234-238).
 
@@ -494,17 +514,20 @@ def load_fasttree_plugin(enable_fasttree=True, annotate_breakdown=False):
             self.model_config.num_attention_heads, self.model_config.num_key_value_heads,
             self.model_config.head_dim, torch.device("cuda", self.gpu_id))
         self._fasttree_planned_for = None
+        self._fasttree_forwards = 0
 
     ModelTpServer.__init__ = server_init_with_metadata
 
     decode_batch = ModelTpServer.forward_decode_batch
 
+    try:
+        from sglang.global_config import global_config
+        replan_every = int(global_config.num_continue_decode_steps)
+    except Exception:
+        replan_every = 10
+
     def decode_batch_with_plan(self, batch):
-        if same_requests(self._fasttree_planned_for, batch.reqs):
-            this.prepare_for_fasttree_step(batch, self.fasttree_metadata)
-        else:
-            this.prepare_for_fasttree_meta(batch, self.fasttree_metadata)
-            self._fasttree_planned_for = tuple(batch.reqs)
+        plan_or_step(self, batch, replan_every, this.prepare_for_fasttree_meta, this.prepare_for_fasttree_step)
         return decode_batch(self, batch)
 
     ModelTpServer.forward_decode_batch = decode_batch_with_plan

@@ -165,6 +165,11 @@ def _kernel_cases():
               alpha=0.0, beta=0.0, gamma=10.0, kv_split_sizes=(81920, 81920), **big),
         # C1 of the baseline in full: 32/32 heads, root 1024 tokens, 16 leaves of 128
         _case("k_c1", regular([1, 16], [1024, 128]), 32, 32, D=128, dtype="fp16", seed=18),
+        # C2 and C3 of the baseline at full size; the fixtures keep the outputs of every
+        # `keep_every`-th request only (the interpreter still runs the whole launch)
+        dict(_case("k_c2", regular([1, 64], [4096, 256]), 32, 8, D=128, dtype="fp16", seed=19, **big), keep_every=4),
+        dict(_case("k_c3", regular([1, 10, 400], [4000, 400, 40]), 32, 8, D=128, dtype="fp16", seed=20, **big),
+             keep_every=16),
     ]
 
 

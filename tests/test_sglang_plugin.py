@@ -516,3 +516,33 @@ def test_merge_path_hand_derived():
     prepare_for_fasttree_meta(batch, shipped)
     prepare_for_fasttree_meta(batch, same)
     assert plan_lists(same, batch) == plan_lists(shipped, batch)
+
+
+def test_hook_replans_for_new_requests_and_every_few_forwards():
+    """The decision the patched forward_decode_batch takes, with stand-ins for the server and the
+    requests: a new plan for a batch of other request objects -- also when a finished request was
+    freed and a new one may sit at its address --, the +1 step while the batch is unchanged, and
+    a new plan after `replan_every` forwards (the reference plans once per forward_step and steps
+    between its num_continue_decode_steps forwards, plugin.py:108-131)."""
+    import gc
+    from fasttree_hip.sglang_plugin import plan_or_step
+    calls = []
+    plan = lambda batch, meta: calls.append("plan")
+    step = lambda batch, meta: calls.append("step")
+    server = Obj(fasttree_metadata=object(), _fasttree_planned_for=None, _fasttree_forwards=0)
+    a, b = Req([1], []), Req([2], [])
+    batch = Obj(reqs=[a, b])
+    assert [plan_or_step(server, batch, 3, plan, step) for _ in range(7)] == ["plan", "step", "step", "plan", "step", "step", "plan"]
+    batch.reqs = [a]                              # a request finished
+    assert plan_or_step(server, batch, 3, plan, step) == "plan"
+    # batch size 1 served back to back: the old request is freed before the new one is made
+    del a, b
+    batch.reqs = [Req([3], [])]
+    seen = set()
+    for _ in range(50):
+        assert plan_or_step(server, batch, 100, plan, step) == "plan"
+        seen.add(id(batch.reqs[0]))
+        batch.reqs = []                           # the only other holder lets go ...
+        gc.collect()
+        batch.reqs = [Req([4], [])]               # ... and a new request is made, possibly at the same address
+    assert calls.count("plan") == 54 and calls.count("step") == 4
