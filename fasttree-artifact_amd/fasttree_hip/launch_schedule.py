@@ -150,34 +150,36 @@ def _runs_of(kv_offs, kv_lens, q_offs, q_lens, q_entries):
     list and was cut by the planner into chunks of ``chunk_lens`` tokens.
     """
     n = len(kv_offs)
-    order = np.lexsort((q_offs, kv_lens, kv_offs))
+    order = np.lexsort((q_offs, kv_lens, kv_offs)).tolist()
+    # (plain lists: the scan below touches every vnode once, and numpy scalars are slow at that)
+    ko, kl, qo, ql = kv_offs.tolist(), kv_lens.tolist(), q_offs.tolist(), q_lens.tolist()
     chunks = []   # (kv_off, kv_len, requests)
     i = 0
     while i < n:
         v = order[i]
-        reqs = [q_entries[q_offs[v]: q_offs[v] + q_lens[v]]]
-        end = q_offs[v] + q_lens[v]
+        first = qo[v]
+        end = first + ql[v]
         j = i + 1
         while j < n:
             w = order[j]
-            if kv_offs[w] != kv_offs[v] or kv_lens[w] != kv_lens[v] or q_offs[w] != end:
+            if ko[w] != ko[v] or kl[w] != kl[v] or qo[w] != end:
                 break
-            reqs.append(q_entries[q_offs[w]: q_offs[w] + q_lens[w]])
-            end = q_offs[w] + q_lens[w]
+            end += ql[w]
             j += 1
-        chunks.append((int(kv_offs[v]), int(kv_lens[v]), np.concatenate(reqs)))
+        chunks.append((ko[v], kl[v], q_entries[first:end]))   # (the tiles' rows adjoin: one slice)
         i = j
     # chain the chunks of one node: the next chunk starts where this one ends, same requests
+    keys = [reqs.tobytes() for _, _, reqs in chunks]
     by_start = {}
     for idx, (off, length, reqs) in enumerate(chunks):
-        by_start.setdefault(off, []).append(idx)
+        by_start.setdefault((off, keys[idx]), []).append(idx)
     follower = [-1] * len(chunks)
     has_leader = [False] * len(chunks)
     for idx, (off, length, reqs) in enumerate(chunks):
         if length == 0:
             continue
-        for cand in by_start.get(off + length, ()):
-            if cand != idx and not has_leader[cand] and np.array_equal(chunks[cand][2], reqs):
+        for cand in by_start.get((off + length, keys[idx]), ()):
+            if cand != idx and not has_leader[cand]:
                 follower[idx] = cand
                 has_leader[cand] = True
                 break
@@ -203,16 +205,19 @@ def block_programs(kv_offs, kv_lens, q_offs, q_lens, q_entries, batch_size, grou
     start, and a program that has its compute unit to itself steps faster), and the layout with
     the shorter modelled duration is returned.
     """
+    kv_offs, kv_lens, q_offs, q_lens = (np.asarray(x, dtype=np.int64) for x in (kv_offs, kv_lens, q_offs, q_lens))
+    q_entries = np.asarray(q_entries, dtype=np.int64)
+    runs = _runs_of(kv_offs, kv_lens, q_offs, q_lens, q_entries)
     if block_slots is None:
-        both = [_block_programs(kv_offs, kv_lens, q_offs, q_lens, q_entries, batch_size, group, num_kv_heads,
+        both = [_block_programs(runs, batch_size, group, num_kv_heads,
                                 block_rows=block_rows, block_slots=slots, recut=recut, embed=embed, head_dim=head_dim)
                 for slots in (BLOCK_SLOTS, BLOCK_SLOTS // 2)]
         return min(both, key=lambda sched: sched.modelled_us)
-    return _block_programs(kv_offs, kv_lens, q_offs, q_lens, q_entries, batch_size, group, num_kv_heads,
+    return _block_programs(runs, batch_size, group, num_kv_heads,
                            block_rows=block_rows, block_slots=block_slots, recut=recut, embed=embed, head_dim=head_dim)
 
 
-def _block_programs(kv_offs, kv_lens, q_offs, q_lens, q_entries, batch_size, group, num_kv_heads, *,
+def _block_programs(runs, batch_size, group, num_kv_heads, *,
                     block_rows, block_slots, recut, embed, head_dim) -> LaunchSchedule:
     """One layout of :func:`block_programs`, for ``block_slots`` programs at a time.
 
@@ -225,14 +230,11 @@ def _block_programs(kv_offs, kv_lens, q_offs, q_lens, q_entries, batch_size, gro
     has its compute unit to itself steps only about a fifth faster, so narrow vnodes inside the
     programs run one after the other with the wide work all the same.
     """
-    kv_offs, kv_lens, q_offs, q_lens = (np.asarray(x, dtype=np.int64) for x in (kv_offs, kv_lens, q_offs, q_lens))
-    q_entries = np.asarray(q_entries, dtype=np.int64)
     group = max(1, int(group))
     heads = max(1, int(num_kv_heads))
     cap = max(1, int(block_rows) // group)            # requests per row chunk
     per_round = max(1, int(block_slots) // heads)     # programs per round and head
 
-    runs = _runs_of(kv_offs, kv_lens, q_offs, q_lens, q_entries)
     wide_runs, narrow = [], []    # narrow: (kv_off, kv_len, requests) per planner chunk
     for start, lens, reqs in runs:
         rows = len(reqs) * group
