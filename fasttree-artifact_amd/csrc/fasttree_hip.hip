@@ -658,19 +658,24 @@ __device__ __forceinline__ void tile_step32(const WideLane& la, unsigned off, in
   using W = WideGeom<D>;
   constexpr int KS = D / 16, DB = D / 32, NV = 2 * DB;
 
-  // all K operands of the tile are requested before the first contraction needs one
+  // the K operands are requested eight contraction steps at a time, before the first of those
+  // steps needs one (all of them at once up to head_dim 128)
   const unsigned kb = la.k + off;
-  u32x4 kf[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) kf[ks] = lds_read16(kb ^ (32u * ks));
-  // (keeps the scheduler from sinking each read next to its use, which would expose the full
-  // LDS latency eight times in a row)
-  __builtin_amdgcn_sched_barrier(0);
+  constexpr int KB = KS < 8 ? KS : 8;
   f32x16 s;
 #pragma unroll
   for (int j = 0; j < 16; ++j) s[j] = 0.f;
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) s = E::mfma32(kf[ks], qf[ks], s);
+  for (int k0 = 0; k0 < KS; k0 += KB) {
+    u32x4 kf[KB];
+#pragma unroll
+    for (int ks = 0; ks < KB; ++ks) kf[ks] = lds_read16(kb ^ (32u * (k0 + ks)));
+    // (keeps the scheduler from sinking each read next to its use, which would expose the full
+    // LDS latency eight times in a row)
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < KB; ++ks) s = E::mfma32(kf[ks], qf[k0 + ks], s);
+  }
 
   if (valid < kTileTokens) {  // wave uniform
     asm volatile("" ::: "memory");  // keeps this a branch: as selects it would run on every tile
@@ -680,16 +685,19 @@ __device__ __forceinline__ void tile_step32(const WideLane& la, unsigned off, in
   }
 
   // the V^T operands do not depend on the probabilities: request them now, so that they arrive
-  // under the soft-max arithmetic (they take the registers the K operands just left)
+  // under the soft-max arithmetic (they take the registers the K operands just left); at
+  // head_dim 256 only those of the first 16 tokens, the others after the first half of P.V
   const unsigned vlo = la.v_lo + off, vhi = la.v_hi + off;
-  u32x4 vf[NV];
-#pragma unroll
-  for (int i = 0; i < NV; ++i) {
+  constexpr int VH = D > 128 ? DB : NV;   // operands requested ahead of the soft-max
+  u32x4 vf[VH];
+  auto read_v = [&](int i) {
     const int u = i / DB, db = i % DB;
     const u32x2 lo = lds_read_tr8((vlo ^ (64u * db)) + u * 16 * W::kRowBytes);
     const u32x2 hi = lds_read_tr8((vhi ^ (64u * db)) + u * 16 * W::kRowBytes);
-    vf[i] = u32x4{lo[0], lo[1], hi[0], hi[1]};
-  }
+    return u32x4{lo[0], lo[1], hi[0], hi[1]};
+  };
+#pragma unroll
+  for (int i = 0; i < VH; ++i) vf[i] = read_v(i);
   __builtin_amdgcn_sched_barrier(0);
   float mx = max3(s[0], s[1], s[2]);
 #pragma unroll
@@ -722,7 +730,15 @@ __device__ __forceinline__ void tile_step32(const WideLane& la, unsigned off, in
     for (int i = 0; i < 4; ++i) st.l = E::add_pair(pf[u][i], st.l);
 
 #pragma unroll
-  for (int i = 0; i < NV; ++i) st.o[i % DB] = E::mfma32(vf[i], pf[i / DB], st.o[i % DB]);
+  for (int i = 0; i < VH; ++i) st.o[i % DB] = E::mfma32(vf[i], pf[i / DB], st.o[i % DB]);
+  if constexpr (VH < NV) {
+    u32x4 vg[NV - VH];
+#pragma unroll
+    for (int i = VH; i < NV; ++i) vg[i - VH] = read_v(i);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = VH; i < NV; ++i) st.o[i % DB] = E::mfma32(vg[i - VH], pf[i / DB], st.o[i % DB]);
+  }
 }
 
 template <int D>
@@ -1310,7 +1326,7 @@ __device__ __forceinline__ int wide_vnode_of_rank(const Stage1Args& a, char* sme
 // (blocks that stream the same KV run are launched together and share it in L2); the narrow
 // blocks follow and fill the machine while the wide blocks drain.
 template <typename E, int D, bool GATHERED>
-__global__ void __launch_bounds__(kWideBlock, 512 / kWideBlock) stage1_fused_kernel(Stage1Args a) {
+__global__ void __launch_bounds__(kWideBlock, D > 128 ? 1 : 512 / kWideBlock) stage1_fused_kernel(Stage1Args a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int wide_blocks = a.prog_table ? a.num_programs * a.hkv : a.vnode_count * a.wide_chunks * a.hkv;
   const int wide_index = blockIdx.x, narrow_index = (int)blockIdx.x - wide_blocks;
@@ -1530,8 +1546,8 @@ inline int wave_slots() {
   }
   return slots;
 }
-inline int narrow_share_for(int64_t items) {
-  const int slots = wave_slots();
+inline int narrow_share_for(int64_t items, int head_dim) {
+  const int slots = head_dim > 128 ? wave_slots() / 2 : wave_slots();   // (one block per compute unit at 512-byte rows)
   int share = 1;
   while (share < kWideWaves && 4 * items * (2 * share) <= 3 * (int64_t)slots) share *= 2;
   return share;
@@ -1554,11 +1570,11 @@ int launch_stage1_fused(const Stage1Args& a0, hipStream_t stream) {
   }
   Stage1Args a = a0;
   const int64_t narrow_items = (int64_t)(a.narrow_count - a.narrow_in_programs) * a.hkv;  // those of the trailing blocks
-  a.narrow_share = narrow_share_for(narrow_items);
+  a.narrow_share = narrow_share_for(narrow_items, D);
   const int per_block = kWideWaves / a.narrow_share;
   const int64_t narrow_blocks = (narrow_items + per_block - 1) / per_block;
   a.wide_chunks = std::max(1, std::min(8, (a.wide_rows + kWideRows - 1) / kWideRows));
-  a.block_slots = wave_slots() / kWideWaves;
+  a.block_slots = (D > 128 ? wave_slots() / 2 : wave_slots()) / kWideWaves;
   const int64_t wide_blocks = a.prog_table ? (int64_t)a.num_programs * a.hkv : (int64_t)a.vnode_count * a.wide_chunks * a.hkv;
   const int64_t blocks = wide_blocks + narrow_blocks;
   if (blocks == 0) return FT_OK;
@@ -1573,7 +1589,7 @@ int launch_stage1_narrow(const Stage1Args& a0, hipStream_t stream) {
   const int64_t blocks = (int64_t)a.narrow_count * a.hkv;
   if (blocks == 0) return FT_OK;
   if (blocks > INT32_MAX) return FT_ERR_ARGUMENT;
-  a.narrow_share = narrow_share_for(blocks);
+  a.narrow_share = narrow_share_for(blocks, D);
   auto kern = stage1_narrow_kernel<E, D, GATHERED>;
   const size_t lds = (size_t)a.narrow_share * NarrowGeom<D>::kLds;
   static bool configured_on[kMaxDevices] = {};  // raising the dynamic LDS limit is idempotent
@@ -1592,7 +1608,7 @@ int launch_stage1_narrow(const Stage1Args& a0, hipStream_t stream) {
 
 // `a` names two vnode ranges: [vnode_begin, +vnode_count) of wide vnodes (more than 16 query
 // rows) and [narrow_begin, +narrow_count) of narrow ones.
-template <typename E, int D, bool GATHERED, bool STAGED = (D > 128)>
+template <typename E, int D, bool GATHERED, bool STAGED = false>
 int launch_stage1_d(const Stage1Args& a, hipStream_t stream) {
   if constexpr (STAGED) {
     // 128-token double buffers of 512-byte rows do not fit in LDS: per-wave staging kernels
@@ -1864,7 +1880,7 @@ int ft_stage1_programs(const void* q, const void* k, const void* v,
   if (num_kv_heads < 1 || num_qo_heads % num_kv_heads != 0) return FT_ERR_GROUP;
   const int g = num_qo_heads / num_kv_heads;
   if (int rc = check_common(head_dim, g, dtype)) return rc;
-  if (head_dim < 32 || head_dim > 128) return FT_ERR_HEAD_DIM;  // the program table is for the direct-load kernels
+  if (head_dim < 32) return FT_ERR_HEAD_DIM;  // the program table is for the direct-load kernels
   if (phase_node_nums[0] == 0 && phase_node_nums[1] == 0) return FT_OK;
   Stage1Args a;
   if (int rc = stage1_setup(a, q, k, v, sq0, sq1, sk0, sk1, sv0, sv1, vnode_to_kv_entries, vnode_to_kv_offs,

@@ -68,7 +68,7 @@ def fasttree_decode(
         raise _lib.FastTreeLibraryError("mid_o and mid_lse must be float32")
     lib = _lib.load()
     programs = getattr(phase_node_nums, "prog_table", None)
-    if programs is not None and 32 <= q.shape[-1] <= 128:
+    if programs is not None and q.shape[-1] >= 32:
         # the launch was arranged as block programs (launch_schedule.block_programs)
         rc = lib.ft_decode_programs(
             q.data_ptr(), k_buffer.data_ptr(), v_buffer.data_ptr(), o.data_ptr(),
@@ -147,7 +147,7 @@ def fasttree_decode_stage1(q, k_buffer, v_buffer, vnode_to_kv_entries, vnode_to_
     _need_gpu(q, k_buffer, v_buffer, mid_o, mid_lse)
     lib = _lib.load()
     programs = getattr(phase_node_nums, "prog_table", None)
-    if programs is not None and 32 <= q.shape[-1] <= 128:
+    if programs is not None and q.shape[-1] >= 32:
         rc = lib.ft_stage1_programs(
             q.data_ptr(), k_buffer.data_ptr(), v_buffer.data_ptr(),
             q.stride(0), q.stride(1), k_buffer.stride(0), k_buffer.stride(1), v_buffer.stride(0), v_buffer.stride(1),

@@ -209,9 +209,11 @@ def block_programs(kv_offs, kv_lens, q_offs, q_lens, q_entries, batch_size, grou
     q_entries = np.asarray(q_entries, dtype=np.int64)
     runs = _runs_of(kv_offs, kv_lens, q_offs, q_lens, q_entries)
     if block_slots is None:
+        # (at head_dim 256 a compute unit holds one block of the kernel: 512-byte rows, 136 KB of LDS)
+        layouts = (BLOCK_SLOTS, BLOCK_SLOTS // 2) if head_dim <= 128 else (BLOCK_SLOTS // 2,)
         both = [_block_programs(runs, batch_size, group, num_kv_heads,
                                 block_rows=block_rows, block_slots=slots, recut=recut, embed=embed, head_dim=head_dim)
-                for slots in (BLOCK_SLOTS, BLOCK_SLOTS // 2)]
+                for slots in layouts]
         return min(both, key=lambda sched: sched.modelled_us)
     return _block_programs(runs, batch_size, group, num_kv_heads,
                            block_rows=block_rows, block_slots=block_slots, recut=recut, embed=embed, head_dim=head_dim)

@@ -525,7 +525,7 @@ def fasttree_preparation(
     phase_nums, phase_offs = list(plan.phase_node_nums), list(plan.phase_node_offsets)
     if launch_order:
         group = max(1, num_qo_heads // num_kv_heads)
-        sched = block_programs(*vnodes, q_entries, batch_size, group, num_kv_heads)
+        sched = block_programs(*vnodes, q_entries, batch_size, group, num_kv_heads, head_dim=head_dim)
         vnodes = (sched.kv_offs, sched.kv_lens, sched.q_offs, sched.q_lens)
         q_entries = sched.q_entries
         per_request = (sched.req_entries, sched.req_offs, sched.req_lens)

@@ -131,7 +131,7 @@ int ft_decode(const void* q, const void* k, const void* v, void* o,
  * before the others instead of after them).  The first narrow_in_programs vnodes of the second
  * range belong to programs; the rest of it is served one wave each by blocks of their own, as in
  * ft_stage1_phases, whatever their width.  The lists are otherwise those of ft_decode and
- * describe a complete plan without the table.  head_dim in {32, 64, 128}.  The table is
+ * describe a complete plan without the table.  head_dim in {32, 64, 128, 256}.  The table is
  * trusted: it is not read on the host.
  */
 int ft_stage1_programs(const void* q, const void* k, const void* v,

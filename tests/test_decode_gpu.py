@@ -485,7 +485,7 @@ def test_more_wide_vnodes_than_the_ranking_holds(device):
 def test_light_wide_vnodes_run_with_the_narrow_phase_at_every_head_size(d, device):
     """More first-phase blocks than the device holds, all of them light (32-64 rows x 20-30
     tokens): the launch order hands them to the narrow path, which serves them in passes of 16
-    rows (head_dim 256 goes through the register-staged kernel, without the program table)."""
+    rows (head_dim 256: one block per compute unit, the programs are laid out on 256 block slots)."""
     _announce("light wide vnodes", d)
     aux = _plan_and_check(device, [1, 150, 1200], [20, 30, 9], 16, 4, d, [16, 4], [1024, 128], f"light wide d{d}",
                           sample=list(range(0, 1200, 23)), thr=((132, 528), (132, 132)))
