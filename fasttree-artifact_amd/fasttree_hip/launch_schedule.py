@@ -214,14 +214,15 @@ def block_programs(kv_offs, kv_lens, q_offs, q_lens, q_entries, batch_size, grou
         both = [_block_programs(runs, batch_size, group, num_kv_heads,
                                 block_rows=block_rows, block_slots=slots, recut=recut, embed=embed, head_dim=head_dim)
                 for slots in layouts]
-        return min(both, key=lambda sched: sched.modelled_us)
+        return min(both, key=lambda layout: layout[0])[1]()     # (only the chosen layout's lists are built)
     return _block_programs(runs, batch_size, group, num_kv_heads,
-                           block_rows=block_rows, block_slots=block_slots, recut=recut, embed=embed, head_dim=head_dim)
+                           block_rows=block_rows, block_slots=block_slots, recut=recut, embed=embed, head_dim=head_dim)[1]()
 
 
 def _block_programs(runs, batch_size, group, num_kv_heads, *,
-                    block_rows, block_slots, recut, embed, head_dim) -> LaunchSchedule:
-    """One layout of :func:`block_programs`, for ``block_slots`` programs at a time.
+                    block_rows, block_slots, recut, embed, head_dim):
+    """One layout of :func:`block_programs`, for ``block_slots`` programs at a time: its
+    modelled duration and a function that builds its :class:`LaunchSchedule`.
 
     Takes the four per-vnode lists and the scratch-row list of kernel_bench/fasttree.py:193-231
     (any order), the number of requests, the GQA group size and the number of KV heads.
@@ -370,40 +371,6 @@ def _block_programs(runs, batch_size, group, num_kv_heads, *,
     taken = {id(v) for v in embedded}
     narrow = embedded + [v for v in narrow if id(v) not in taken]
 
-    # ---- the lists: wide pieces in program order, then the narrow vnodes
-    new_kv_offs, new_kv_lens, new_q_offs, new_q_lens, rows_out = [], [], [], [], []
-    prog_table = []
-    row = 0
-
-    def emit(off, length, reqs):
-        nonlocal row
-        new_kv_offs.append(off)
-        new_kv_lens.append(length)
-        new_q_offs.append(row)
-        new_q_lens.append(len(reqs))
-        rows_out.append(reqs)
-        row += len(reqs)
-
-    narrow_first = 0
-    for p, prog in enumerate(programs):
-        wide_first = len(new_kv_offs)
-        for i in prog:
-            emit(*pieces[i][:3])
-        # the two blocks of a compute unit (block b and b + 256) get opposite orders
-        front = (p % per_round) < per_round // 2
-        prog_table.append((wide_first, len(new_kv_offs), narrow_first, -len(shares[p]) if front else len(shares[p])))
-        narrow_first += len(shares[p])
-    n_wide = len(new_kv_offs)
-    for off, length, reqs in narrow:
-        emit(off, length, reqs)
-    new_q_entries = np.concatenate(rows_out) if rows_out else np.zeros(0, dtype=np.int64)
-
-    # scratch rows of every request, in row order (kernel_bench/fasttree.py:233-244)
-    by_req = np.argsort(new_q_entries, kind="stable")
-    req_lens = np.bincount(new_q_entries, minlength=int(batch_size)).astype(np.int64)[: int(batch_size)]
-    req_offs = np.concatenate([[0], np.cumsum(req_lens)[:-1]]) if batch_size else np.zeros(0, dtype=np.int64)
-    req_entries = np.concatenate([by_req, np.full(32, -1, dtype=np.int64)])
-
     # ---- modelled duration of the launch (microseconds)
     shared = len(programs) * heads > BLOCK_SLOTS // 2          # two program blocks on some compute unit
     tile_us = TILE_US_SHARED if shared else TILE_US_ALONE
@@ -412,6 +379,7 @@ def _block_programs(runs, batch_size, group, num_kv_heads, *,
         wide_us = max(max(program_tiles), sum(program_tiles) / len(programs) * waves_of_blocks) * tile_us
     else:
         wide_us = 0.0
+    narrow_first = sum(len(sh) for sh in shares)
     trailing = narrow[narrow_first:]
     if trailing:
         item_us = [narrow_work(v) * TILE_US_SHARED for v in trailing]
@@ -425,12 +393,49 @@ def _block_programs(runs, batch_size, group, num_kv_heads, *,
     else:
         modelled = wide_us
 
-    i32 = lambda x: np.asarray(x, dtype=np.int32)
-    return LaunchSchedule(
-        kv_offs=i32(new_kv_offs), kv_lens=i32(new_kv_lens), q_offs=i32(new_q_offs), q_lens=i32(new_q_lens),
-        q_entries=i32(new_q_entries), req_entries=i32(req_entries), req_offs=i32(req_offs), req_lens=i32(req_lens),
-        phase_node_nums=[n_wide, len(new_kv_offs) - n_wide], phase_node_offsets=[0, n_wide],
-        prog_table=i32(prog_table).reshape(-1, 4), narrow_in_programs=narrow_first,
-        program_tiles=np.asarray(program_tiles, dtype=np.float64), block_slots=int(block_slots),
-        modelled_us=float(modelled),
-    )
+    def build() -> LaunchSchedule:
+        # ---- the lists: wide pieces in program order, then the narrow vnodes
+        new_kv_offs, new_kv_lens, new_q_offs, new_q_lens, rows_out = [], [], [], [], []
+        prog_table = []
+        row = 0
+
+        def emit(off, length, reqs):
+            nonlocal row
+            new_kv_offs.append(off)
+            new_kv_lens.append(length)
+            new_q_offs.append(row)
+            new_q_lens.append(len(reqs))
+            rows_out.append(reqs)
+            row += len(reqs)
+
+        narrow_first = 0
+        for p, prog in enumerate(programs):
+            wide_first = len(new_kv_offs)
+            for i in prog:
+                emit(*pieces[i][:3])
+            # the two blocks of a compute unit (block b and b + 256) get opposite orders
+            front = (p % per_round) < per_round // 2
+            prog_table.append((wide_first, len(new_kv_offs), narrow_first, -len(shares[p]) if front else len(shares[p])))
+            narrow_first += len(shares[p])
+        n_wide = len(new_kv_offs)
+        for off, length, reqs in narrow:
+            emit(off, length, reqs)
+        new_q_entries = np.concatenate(rows_out) if rows_out else np.zeros(0, dtype=np.int64)
+
+        # scratch rows of every request, in row order (kernel_bench/fasttree.py:233-244)
+        by_req = np.argsort(new_q_entries, kind="stable")
+        req_lens = np.bincount(new_q_entries, minlength=int(batch_size)).astype(np.int64)[: int(batch_size)]
+        req_offs = np.concatenate([[0], np.cumsum(req_lens)[:-1]]) if batch_size else np.zeros(0, dtype=np.int64)
+        req_entries = np.concatenate([by_req, np.full(32, -1, dtype=np.int64)])
+
+        i32 = lambda x: np.asarray(x, dtype=np.int32)
+        return LaunchSchedule(
+            kv_offs=i32(new_kv_offs), kv_lens=i32(new_kv_lens), q_offs=i32(new_q_offs), q_lens=i32(new_q_lens),
+            q_entries=i32(new_q_entries), req_entries=i32(req_entries), req_offs=i32(req_offs), req_lens=i32(req_lens),
+            phase_node_nums=[n_wide, len(new_kv_offs) - n_wide], phase_node_offsets=[0, n_wide],
+            prog_table=i32(prog_table).reshape(-1, 4), narrow_in_programs=narrow_first,
+            program_tiles=np.asarray(program_tiles, dtype=np.float64), block_slots=int(block_slots),
+            modelled_us=float(modelled),
+        )
+
+    return float(modelled), build

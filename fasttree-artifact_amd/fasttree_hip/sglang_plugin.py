@@ -340,16 +340,16 @@ def prepare_for_fasttree_meta(batch, fasttree_metadata: FastTreeMetadata):
         tail_ends = [lists[0][v] + lists[1][v] for v in meta.req_last_vnodes]
         sched = block_programs(*lists, q_entries, len(batch.reqs), meta.kv_group_num, meta.num_kv_heads,
                                head_dim=meta.head_dim)
-        lists = [x.tolist() for x in (sched.kv_offs, sched.kv_lens, sched.q_offs, sched.q_lens)]
-        q_entries = sched.q_entries.tolist()
-        req_entries = sched.req_entries[: sched.num_rows].tolist()
-        req_offs, req_lens = sched.req_offs.tolist(), sched.req_lens.tolist()
+        lists = [sched.kv_offs, sched.kv_lens, sched.q_offs, sched.q_lens]      # (int32 arrays, uploaded as they are)
+        q_entries = sched.q_entries
+        req_entries = sched.req_entries[: sched.num_rows]
+        req_offs, req_lens = sched.req_offs, sched.req_lens
         # a request's last vnode is the single-request vnode that ends where its tokens end
         # (narrow vnodes keep the planner's chunks, so there is exactly one)
-        ends_of = {}
-        for v, (ko, kl, qo, ql) in enumerate(zip(*lists)):
-            if ql == 1:
-                ends_of[(ko + kl, q_entries[qo])] = v
+        single = np.flatnonzero(sched.q_lens == 1)
+        ends = (sched.kv_offs[single].astype(np.int64) + sched.kv_lens[single]).tolist()
+        owner = sched.q_entries[sched.q_offs[single]].tolist()
+        ends_of = dict(zip(zip(ends, owner), single.tolist()))
         meta.req_last_vnodes = [ends_of[(end, rid)] for rid, end in enumerate(tail_ends)]
         nums = LaunchPhases(sched.phase_node_nums)
         if sched.num_programs > 0:
@@ -365,7 +365,10 @@ def prepare_for_fasttree_meta(batch, fasttree_metadata: FastTreeMetadata):
         meta.phase_node_nums, meta.phase_node_offsets = nums, list(sched.phase_node_offsets)
 
     def upload(dst, values):
-        src = torch.tensor(values, device="cpu", dtype=torch.int32)
+        if isinstance(values, np.ndarray):
+            src = torch.from_numpy(np.ascontiguousarray(values, dtype=np.int32))
+        else:
+            src = torch.tensor(values, device="cpu", dtype=torch.int32)
         dst[: src.numel()].copy_(src, non_blocking=True)
 
     upload(meta.vnode_to_q_entries, q_entries)
