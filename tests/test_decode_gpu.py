@@ -416,7 +416,7 @@ def test_runs_cut_anew_into_block_programs(device, monkeypatch):
     cut into equal programs (pieces at multiples of 64 tokens instead of the planner's two
     chunks); same result as with the planner's own lists, both at the parity bar.  Then forced
     on a small three-level tree (every run cut anew, every program of several vnodes), fp16 and
-    bf16, on all block slots and on half of them."""
+    bf16, on all block slots and on half of them, as packed programs and with a block per piece."""
     from fasttree_hip import launch_schedule
     _announce("block programs")
     sample = list(range(0, 1024, 41))
@@ -426,19 +426,26 @@ def test_runs_cut_anew_into_block_programs(device, monkeypatch):
     ref = _plan_and_check(device, [1, 1024], [2048, 32], 32, 8, 128, [16, 4], [1024, 256], "kv chunks as planned",
                           sample=sample, thr=((256, 1024), (256, 256)), launch_order=False)
     assert ref[8].tolist() == [3] * 1024
+    aux = _plan_and_check(device, [1, 10, 400], [4000, 400, 40], 32, 8, 128, [16, 4], [1024, 256], "a block per piece",
+                          sample=list(range(0, 400, 13)), thr=((256, 1024), (256, 256)))
+    table = aux[11].prog_table.cpu().view(-1, 4)
+    assert aux[11].num_programs == 59 and int((table[:, 1] - table[:, 0]).max()) == 1, "every piece has its own program"
+    monkeypatch.setattr(launch_schedule, "RESIDENT_MARGIN", 0.0)     # the packed layout
     aux = _plan_and_check(device, [1, 10, 400], [4000, 400, 40], 32, 8, 128, [16, 4], [1024, 256], "programs of several vnodes",
                           sample=list(range(0, 400, 13)), thr=((256, 1024), (256, 256)))
     table = aux[11].prog_table.cpu().view(-1, 4)
     assert int((table[:, 1] - table[:, 0]).max()) > 1, "programs of several vnodes"
     monkeypatch.setattr(launch_schedule, "MIN_PROGRAM_TILES", 0.0)
     monkeypatch.setattr(launch_schedule, "MIN_PIECE_TOKENS", 64)
-    for slots in (512, 256, 4):
-        monkeypatch.setattr(launch_schedule, "BLOCK_SLOTS", slots)
-        for dtype in (torch.float16, torch.bfloat16):
-            aux = _plan_and_check(device, [1, 4, 36], [700, 300, 45], 16, 4, 128, [16, 4], [256, 64],
-                                  f"programs forced {slots} {dtype}", dtype=dtype, thr=((10**6, 10**6), (1, 1)))
-            table = aux[11].prog_table.cpu().view(-1, 4)
-            assert aux[11].num_programs > 0 and int(table[-1, 1]) == aux[11][0]
+    for margin in (0.0, 10.0):                                       # packed programs; a block per piece wherever it exists
+        monkeypatch.setattr(launch_schedule, "RESIDENT_MARGIN", margin)
+        for slots in (512, 256, 4):
+            monkeypatch.setattr(launch_schedule, "BLOCK_SLOTS", slots)
+            for dtype in (torch.float16, torch.bfloat16):
+                aux = _plan_and_check(device, [1, 4, 36], [700, 300, 45], 16, 4, 128, [16, 4], [256, 64],
+                                      f"programs forced {slots} {margin} {dtype}", dtype=dtype, thr=((10**6, 10**6), (1, 1)))
+                table = aux[11].prog_table.cpu().view(-1, 4)
+                assert aux[11].num_programs > 0 and int(table[-1, 1]) == aux[11][0]
 
 
 @pytest.mark.gpu

@@ -19,6 +19,8 @@ VARIANTS = {
     "narrow_in_programs_auto": dict(embed=None),
     "one_block_per_unit": dict(block_slots=256),
     "two_blocks_per_unit": dict(block_slots=512, recut=True),
+    "packed": dict(layout="packed"),
+    "resident": dict(layout="resident"),
 }
 
 
@@ -102,7 +104,7 @@ def test_headline_tree_is_cut_into_equal_programs():
     slots / 8 heads) whose modelled work differs by a few percent; pieces start and end at
     multiples of 64 tokens of their run; the 400 leaves stay as the planner made them."""
     case = next(c for c in PLANNER_CASES if c["name"] == "c3")
-    plan, batch, group, s = _schedule(case, block_slots=512)
+    plan, batch, group, s = _schedule(case, block_slots=512, layout="packed")
     assert 56 <= s.num_programs <= 64
     assert s.program_tiles.max() <= 1.1 * s.program_tiles.mean()
     n_wide, n_narrow = s.phase_node_nums
@@ -119,6 +121,31 @@ def test_headline_tree_is_cut_into_equal_programs():
         pieces.sort()
         assert pieces[0][0] == 0 and sum(n for _, n in pieces) == 4000
         assert all(a + n == b for (a, n), (b, _) in zip(pieces, pieces[1:]))
+
+
+def test_headline_tree_gets_a_block_per_piece_when_all_fit():
+    """C3 by default: every (run, row chunk) has programs of its own, all resident from the start
+    (at most 64 per kv head).  The root is cut into as many equal pieces as still fit -- three,
+    at the same multiples of 64 tokens for all 13 row chunks -- the ten 400-token nodes stay
+    whole, programs are listed longest first, and the modelled duration is within
+    RESIDENT_MARGIN of the packed layout's."""
+    case = next(c for c in PLANNER_CASES if c["name"] == "c3")
+    plan, batch, group, s = _schedule(case)
+    packed = _schedule(case, layout="packed")[3]
+    assert s.block_slots == 512 and s.num_programs == 13 * 3 + 20 == s.phase_node_nums[0]
+    assert (s.prog_table[:, 1] - s.prog_table[:, 0] == 1).all() and (s.prog_table[:, 3] == 0).all()
+    assert (np.diff(s.program_tiles) <= 0).all()
+    assert s.modelled_us <= ls.RESIDENT_MARGIN * packed.modelled_us
+    n_wide = s.phase_node_nums[0]
+    root = sorted({(int(o), int(n)) for o, n in zip(s.kv_offs[:n_wide], s.kv_lens[:n_wide]) if o < 4000})
+    assert root == [(0, 1344), (1344, 1344), (2688, 1312)]
+    rest = sorted({(int(o), int(n)) for o, n in zip(s.kv_offs[:n_wide], s.kv_lens[:n_wide]) if o >= 4000})
+    assert rest == [(4000 + 400 * i, 400) for i in range(10)]
+    assert s.num_rows == 400 * 5 < packed.num_rows          # three root rows, one node row, one leaf row a request
+    # a tree whose wide work items outnumber the programs of a round has no such layout
+    c5 = next(c for c in PLANNER_CASES if c["name"] == "c5_seed0")
+    a, b = _schedule(c5)[3], _schedule(c5, layout="packed")[3]
+    assert a.num_programs == b.num_programs and np.array_equal(a.kv_offs, b.kv_offs)
 
 
 def test_small_launches_keep_the_planner_chunks():
