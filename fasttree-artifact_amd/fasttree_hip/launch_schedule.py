@@ -30,7 +30,7 @@ that the second stage merges -- arranged for the machine:
     either filled one after the other with the runs cut wherever a program is full, or -- when
     that leaves the fullest program about as full -- from runs cut into equal pieces that are
     dealt longest first to the least loaded program (measured on an irregular tree of 500
-    requests: 6 % shorter, 14 % fewer vnodes).  All programs end together and the narrow
+    requests: 6 % shorter, 12 % fewer vnodes).  All programs end together and the narrow
     vnodes follow.
 
   The resident layout is taken when it exists and its modelled duration is within

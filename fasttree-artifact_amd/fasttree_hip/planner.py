@@ -493,7 +493,7 @@ def fasttree_preparation(
     ``buffers`` (a :class:`PlanBuffers`) nothing is allocated on the device: the arrays are
     written into its buffers and the returned tensors are their leading parts.  With
     ``launch_order=True`` the lists come back arranged for an MI355X instead
-    (:func:`launch_schedule.block_programs`: the same computation as equal-work block programs,
+    (:func:`launch_schedule.block_programs`: the same computation as block programs,
     with scratch rows and per-request lists of its own); ``phase_node_nums`` is then a list that
     also carries the program table, which ``fasttree_decode`` picks up.
     """

@@ -335,7 +335,7 @@ def prepare_for_fasttree_meta(batch, fasttree_metadata: FastTreeMetadata):
     if getattr(meta, "launch_order", False):
         from .launch_schedule import LaunchPhases, block_programs
 
-        # the same computation as equal-work block programs: long shared runs (a system prompt
+        # the same computation as block programs: long shared runs (a system prompt
         # under a large batch) cut where the machine is full instead of at the KV split
         tail_ends = [lists[0][v] + lists[1][v] for v in meta.req_last_vnodes]
         sched = block_programs(*lists, q_entries, len(batch.reqs), meta.kv_group_num, meta.num_kv_heads,
