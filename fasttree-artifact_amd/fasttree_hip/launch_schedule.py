@@ -75,6 +75,10 @@ TILE_US_SHARED = 1.19
 TILE_US_ALONE = 0.95
 #: Bytes per microsecond the narrow vnodes stream at most (rows of 2 * head_dim bytes at random slots).
 NARROW_BYTES_PER_US = 5.6e6
+#: A tile step of a piece of at most 64 query rows, relative to one of a full block.  The block's
+#: waves then split the tokens of a super tile, but the super tile is loaded all the same: fitted on
+#: the programs of an irregular tree of 500 requests, 1.21 against 1.44 us per tile step.
+LIGHT_TILE_WEIGHT = 0.85
 #: Waves the machine holds (narrow vnodes in flight).
 WAVE_SLOTS = 2048
 #: Waves of a block (each serves one narrow vnode at a time).
@@ -146,7 +150,7 @@ def _tile_weight(rows: int) -> float:
     """Share of a block's time one tile step of a piece with ``rows`` query rows takes: the
     block's four waves form row groups of 32 rows; with half of them idle they split the tokens
     of a 64-token super tile instead (two ways: a super tile holds two tile steps)."""
-    return 1.0 if rows > 64 else 0.55
+    return 1.0 if rows > 64 else LIGHT_TILE_WEIGHT
 
 
 def _row_chunks(n_requests: int, cap: int):
