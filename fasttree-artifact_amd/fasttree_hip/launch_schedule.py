@@ -94,6 +94,16 @@ CUT_TOKENS = 64
 MIN_PIECE_TOKENS = 128
 #: The resident layout is taken when its modelled duration is within this factor of the packed one's.
 RESIDENT_MARGIN = 1.05
+#: Of two program blocks on one compute unit the one launched later steps this much slower (its
+#: waves are the younger on every SIMD and issue second): measured on the 3-level tree, 1.30 against
+#: 1.13 us per tile step; and microseconds per tile step of the older one.
+YOUNGER_BLOCK_SLOWDOWN = 1.15
+TILE_US_OLDER = 1.10
+#: Where pieces of the longest run have to be younger blocks, one piece of every row chunk is made
+#: this much shorter than the others (1 / YOUNGER_BLOCK_SLOWDOWN: the two blocks of such a compute
+#: unit then end together).  Measured on the 3-level tree against equal pieces: stage 1 59.0 ->
+#: 56.2 us, wall per call 70.6 -> 67.3 us, cold call unchanged; 0.8 gives the same.
+SHORT_PIECE_RATIO = 0.87
 #: Equal pieces dealt to the programs are taken when the fullest program is within this factor of the
 #: fullest of the programs filled one after the other.
 DEALT_MARGIN = 1.06
@@ -250,7 +260,7 @@ def block_programs(kv_offs, kv_lens, q_offs, q_lens, q_entries, batch_size, grou
                            layout=layout, cuts=cuts)[1]()
 
 
-def _resident_pieces(items, per_round, tiles):
+def _resident_pieces(items, per_round, tiles, first_row):
     """The wide work as one program per piece, all of them on the machine from the start.
 
     Every (run, row chunk) item starts as one piece.  While the programs number at most
@@ -277,13 +287,26 @@ def _resident_pieces(items, per_round, tiles):
             break
         cuts[key] += 1
         count += len(runs[key])
+    # The programs beyond the first `first_row` share their compute units with the longest ones
+    # and, being the younger blocks there, step about YOUNGER_BLOCK_SLOWDOWN times slower.  When
+    # pieces of the longest run would be among them, that run gets one shorter piece per row
+    # chunk (SHORT_PIECE_RATIO of the others, which grow a little): sorted by length, the short
+    # ones are the younger.
+    longest = max(runs, key=piece_tiles)
+    uneven = (SHORT_PIECE_RATIO < 1.0 and cuts[longest] >= 2 and count > first_row
+              and cuts[longest] * len(runs[longest]) > first_row)
     pieces = []
     for (start, length), members in runs.items():
         n = cuts[(start, length)]
         units = -(-length // CUT_TOKENS)
+        shares = [units // n + (1 if j < units % n else 0) for j in range(n)]
+        if uneven and (start, length) == longest:
+            short = max(MIN_PIECE_TOKENS // CUT_TOKENS, int(round(units * SHORT_PIECE_RATIO / (n - 1 + SHORT_PIECE_RATIO))))
+            rest = units - short
+            shares = [rest // (n - 1) + (1 if j < rest % (n - 1) else 0) for j in range(n - 1)] + [short]
         bounds, done = [], 0
-        for j in range(n):
-            take = min((units // n + (1 if j < units % n else 0)) * CUT_TOKENS, length - done)
+        for share in shares:
+            take = min(share * CUT_TOKENS, length - done)
             if take > 0:
                 bounds.append((start + done, take))
                 done += take
@@ -430,7 +453,7 @@ def _block_programs(runs, batch_size, group, num_kv_heads, *,
             if cuts == "dealt" or d_max <= DEALT_MARGIN * max(load for _, load in filled):
                 pieces, programs = d_pieces, d_programs
         if layout != "packed":
-            resident = _resident_pieces(items, per_round, tiles)
+            resident = _resident_pieces(items, per_round, tiles, max(1, (BLOCK_SLOTS // 2) // heads))
     elif items:
         # The planner's chunks as they are, one vnode per program, longest first.  While the
         # launch would leave half of the machine idle, row chunks are halved (down to 64 rows):
@@ -504,7 +527,13 @@ def _block_programs(runs, batch_size, group, num_kv_heads, *,
                 # unequal programs end one after the other and the trailing blocks take their slots
                 # while the longest still run: the launch lasts as long as its longest program, or
                 # as long as all the work takes on all the slots
-                modelled = max(max(program_tiles) * tile_us,
+                first_row = max(1, (BLOCK_SLOTS // 2) // heads)      # programs that are the older block of their unit
+                if shared:
+                    longest_us = max(t * TILE_US_OLDER * (YOUNGER_BLOCK_SLOWDOWN if i >= first_row else 1.0)
+                                     for i, t in enumerate(program_tiles))
+                else:
+                    longest_us = max(program_tiles) * tile_us
+                modelled = max(longest_us,
                                sum(program_tiles) * heads / float(block_slots) * tile_us + narrow_us(WAVE_SLOTS))
             else:
                 modelled = wide_us + narrow_us(WAVE_SLOTS) if shared else max(wide_us, narrow_us(slots_for_narrow))

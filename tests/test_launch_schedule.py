@@ -126,8 +126,8 @@ def test_headline_tree_is_cut_into_equal_programs():
 def test_headline_tree_gets_a_block_per_piece_when_all_fit():
     """C3 by default: every (run, row chunk) has programs of its own, all resident from the start
     (at most 64 per kv head).  The root is cut into as many equal pieces as still fit -- three,
-    at the same multiples of 64 tokens for all 13 row chunks -- the ten 400-token nodes stay
-    whole, programs are listed longest first, and the modelled duration is within
+    at the same multiples of 64 tokens for all 13 row chunks, one of them shorter (the pieces that
+    end up as the younger block of a compute unit) -- the ten 400-token nodes stay whole, programs are listed longest first, and the modelled duration is within
     RESIDENT_MARGIN of the packed layout's."""
     case = next(c for c in PLANNER_CASES if c["name"] == "c3")
     plan, batch, group, s = _schedule(case)
@@ -138,7 +138,12 @@ def test_headline_tree_gets_a_block_per_piece_when_all_fit():
     assert s.modelled_us <= ls.RESIDENT_MARGIN * packed.modelled_us
     n_wide = s.phase_node_nums[0]
     root = sorted({(int(o), int(n)) for o, n in zip(s.kv_offs[:n_wide], s.kv_lens[:n_wide]) if o < 4000})
-    assert root == [(0, 1344), (1344, 1344), (2688, 1312)]
+    # three pieces at multiples of 64 tokens, the same for all 13 row chunks; 7 of the 39 have to be
+    # the younger block of a compute unit, so one piece per chunk is about SHORT_PIECE_RATIO of the others
+    assert root == [(0, 1408), (1408, 1408), (2816, 1184)]
+    assert all(o % ls.CUT_TOKENS == 0 for o, _ in root) and sum(n for _, n in root) == 4000
+    assert abs(root[2][1] / root[1][1] - ls.SHORT_PIECE_RATIO) < 0.05
+    assert s.kv_lens[:26].min() >= 1408 and set(s.kv_lens[26:39].tolist()) == {1184}  # the younger blocks (programs 32..38) are short ones
     rest = sorted({(int(o), int(n)) for o, n in zip(s.kv_offs[:n_wide], s.kv_lens[:n_wide]) if o >= 4000})
     assert rest == [(4000 + 400 * i, 400) for i in range(10)]
     assert s.num_rows == 400 * 5 < packed.num_rows          # three root rows, one node row, one leaf row a request
