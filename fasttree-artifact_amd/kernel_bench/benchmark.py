@@ -8,8 +8,11 @@ Engines (``--choice``): ``fasttree`` is the tree decode (planner + the two HIP s
 ``[B, max_seqlen, Hkv, D]`` (the layout of kernel_bench/flash_attn_wrap.py:36-70), here a HIP
 kernel of this library, and it is the result the tree decode is checked against with the
 reference's criterion ``allclose(rtol=1e-2, atol=1e-2)`` (kernel_bench/benchmark.py:216-220).
-The reference's other engines (SGLang Triton, FlashInfer, DeFT) are Triton / CUDA libraries and
-have no counterpart here.
+``DeFT`` is DeFT-Flatten's schedule -- the depth-first token order cut into subtrees of 128 tokens,
+one thread block per (subtree, kv head), kernel_bench/DeFT.py:14-135 and benchmark.py:180-211 --
+run through this library's kernels as block programs (``deft_schedule.py``); it is checked against
+the gathered decode like the tree decode.  The reference's other engines (SGLang Triton,
+FlashInfer) are Triton / CUDA libraries and have no counterpart here.
 
 Timing follows the method of ``triton.testing.do_bench`` as the reference calls it
 (kernel_bench/benchmark.py:35,59): per-call device events, a 256 MB buffer cleared before every
@@ -35,6 +38,7 @@ from fasttree_hip.decode import fasttree_decode, gathered_decode  # noqa: E402
 from fasttree_hip.inputs import qkv_preparation  # noqa: E402
 from fasttree_hip.kv_tree import retrive_from_file  # noqa: E402
 from fasttree_hip.planner import FastTreeParams, fasttree_preparation  # noqa: E402
+from deft_schedule import deft_preparation  # noqa: E402
 
 QUANTILES = [0.5, 0.2, 0.8]
 
@@ -158,6 +162,23 @@ def main(args):
 
         out_tree_attn = run_and_bench(call_tree_attn, "fasttree attn").cpu()
 
+    out_deft_attn = None
+    if args.choice in ["DeFT", "all"]:
+        subtree_len = 128  # (kernel_bench/benchmark.py:183)
+        deft_aux = deft_preparation(tree_info, KV_ptrs, batch_size, num_qo_heads, num_kv_heads, head_dim, subtree_len)
+        out_deft = torch.empty(batch_size, num_qo_heads, head_dim, device="cuda", dtype=dtype)
+
+        def call_deft_attn():
+            fasttree_decode(Q, K_tree_tensor, V_tree_tensor, out_deft, *deft_aux, [1, 1], [32, 32], sm_scale)
+            return out_deft
+
+        out_deft_attn = run_and_bench(call_deft_attn, "DeFT attn").cpu()
+
+    if out_flash_attn is not None and out_deft_attn is not None:
+        ok = torch.allclose(out_flash_attn, out_deft_attn, rtol=1e-2, atol=1e-2)
+        print("DeFT attn Check passed!" if ok else "DeFT attn Check failed!", flush=True)
+        results["deft_check"] = bool(ok)
+
     if out_flash_attn is not None and out_tree_attn is not None:
         ok = torch.allclose(out_flash_attn, out_tree_attn, rtol=1e-2, atol=1e-2)
         print("fasttree attn Check passed!" if ok else "fasttree attn Check failed!", flush=True)
@@ -186,7 +207,7 @@ def build_parser():
     parser.add_argument("--num_kv_heads", type=int, default=32)
     parser.add_argument("--head_dim", type=int, default=128)
     parser.add_argument("--signature", type=str, default=None)
-    parser.add_argument("--choice", type=str, choices=["flash_attn", "fasttree", "all"], default="all")
+    parser.add_argument("--choice", type=str, choices=["flash_attn", "fasttree", "DeFT", "all"], default="all")
     parser.add_argument("--profile", action="store_true", default=False)
     parser.add_argument("--mi355x", action="store_true", default=False,
                         help="query tiles, parallelism thresholds and KV split sizes for MI355X instead of the H100 defaults, "
