@@ -326,6 +326,7 @@ def _block_programs(runs, batch_size, group, num_kv_heads, *,
     (any order), the number of requests, the GQA group size and the number of KV heads.
     ``recut`` forces (True) or forbids (False) cutting the wide runs anew; by default they are
     cut anew when every program of one round gets at least :data:`MIN_PROGRAM_TILES` of work.
+    ``layout`` and ``cuts`` force one of the arrangements (see :func:`block_programs`).
     ``embed`` deals the narrow vnodes to the programs (None: when the runs were cut anew and no
     program's share outweighs its wide vnodes).  Off by default: measured, a program block that
     has its compute unit to itself steps only about a fifth faster, so narrow vnodes inside the
@@ -381,10 +382,9 @@ def _block_programs(runs, batch_size, group, num_kv_heads, *,
         nprog = per_round * rounds
         items.sort(key=lambda it: -(it[0] * tiles(sum(it[2]))))
 
-        def fill(mean):
-            """Programs filled to their targets one after the other, runs cut where a program is full."""
+        def fill(target):
+            """Programs filled to `target` one after the other, runs cut where a program is full."""
             pieces, programs, current, load = [], [], [], 0.0
-            target = mean
             for w, start, lens, part in items:
                 run_len, done = sum(lens), 0
                 while done < run_len:
