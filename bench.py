@@ -12,9 +12,13 @@ Prints ONE JSON line on stdout:
                on the launch stream, every call preceded by a cache flush (a 1 GiB buffer
                is rewritten, so neither L2 nor the 256 MB Infinity Cache holds the pool:
                inputs are resident in HBM, not in cache) -- the reference's own method
-               (triton.testing.do_bench, kernel_bench/benchmark.py:59) with a larger flush.
+               (triton.testing.do_bench, kernel_bench/benchmark.py:59) with a larger flush;
+               200 such calls whatever --steps is.
   ms_per_step  wall clock of exactly --steps back-to-back calls / steps (warm caches,
-               launch overhead included).
+               launch overhead included), after --warmup untimed calls.  Before those the
+               device is kept busy with the same call for 200 ms (`device_warmup_ms` in the
+               line): its clocks settle only after about 100 ms of work, and --warmup counts
+               calls, not time (do_bench warms up by time, too).
   roofline     the dominant kernel of the call; its duration is the mean over the timed steps
                of the event-to-event time around its launch.
   cpu_baseline the reference's no-sharing formulation (per-request gathered KV, PyTorch
@@ -36,6 +40,8 @@ for extra in ("fasttree-artifact_amd", "oracle", os.path.join("tests", "golden")
     sys.path.insert(0, os.path.join(ROOT, extra))
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+DEVICE_WARMUP_MS = 200.0       # untimed calls before the --warmup steps, until the device's clocks have settled
+COLD_CALLS = 200               # flush + call repetitions behind `value` (their median)
 MFMA_PEAK_TFLOPS = 2500.0      # dense fp16 / bf16
 
 WORKLOADS = {
@@ -216,11 +222,26 @@ def main():
     # the launch stream before, between and after, for the per-kernel durations -- the events
     # themselves cost a few microseconds per step, which must not leak into ms_per_step.
     if args.phase != "both":
+        t_end = time.perf_counter() + DEVICE_WARMUP_MS * 1e-3
+        while time.perf_counter() < t_end:
+            for _ in range(16):
+                stage1()
+            torch.cuda.synchronize()
         for _ in range(args.warmup + args.steps):
             stage1()
         torch.cuda.synchronize()
         log(f"profile-only: {args.warmup + args.steps} stage-1 launches of the {args.phase} phase, vnodes {list(nums)}")
         return
+    # The device's clocks settle only after about 100 ms of continuous work (measured: 68 us per
+    # step in the first 20 ms of a process, 62 us from 100 ms on), and --warmup counts steps, not
+    # time: keep the device busy with the same call for DEVICE_WARMUP_MS first, as
+    # triton.testing.do_bench warms up by time (kernel_bench/benchmark.py:59), then do the
+    # --warmup steps and time exactly --steps.
+    t_end = time.perf_counter() + DEVICE_WARMUP_MS * 1e-3
+    while time.perf_counter() < t_end:
+        for _ in range(16):
+            step()
+        torch.cuda.synchronize()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -252,7 +273,7 @@ def main():
 
     # ---- cold-cache latency per call (events on the launch stream, flush before every call)
     flush = torch.empty(1 << 28, dtype=torch.int32, device=device)     # 1 GiB
-    reps = max(30, min(args.steps, 200))
+    reps = COLD_CALLS
     cold, warm = [], []
     for _ in range(reps):
         flush.zero_()
@@ -371,6 +392,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "device_warmup_ms": DEVICE_WARMUP_MS,
         "ms_per_step": wall_ms,
         "higher_is_better": False,
         "scaling": "weak",
