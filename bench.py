@@ -9,11 +9,14 @@ reference bench (kernel_bench/benchmark.py:88-127).
 
 Prints ONE JSON line on stdout:
   value        median latency of one decode call in microseconds, measured with events
-               on the launch stream, every call preceded by a cache flush (a 1 GiB buffer
-               is rewritten, so neither L2 nor the 256 MB Infinity Cache holds the pool:
-               inputs are resident in HBM, not in cache) -- the reference's own method
-               (triton.testing.do_bench, kernel_bench/benchmark.py:59) with a larger flush;
-               200 such calls whatever --steps is.
+               on the launch stream, every call preceded by a cache flush: a 1 GiB buffer is
+               rewritten and then read, so neither L2 nor the 256 MB Infinity Cache holds the
+               pool (inputs are resident in HBM, not in cache) and the lines they hold
+               instead are clean; 200 such calls whatever --steps is.  The reference's timer
+               (triton.testing.do_bench, kernel_bench/benchmark.py:59) only rewrites its
+               flush buffer: the call after it also pays for writing the buffer's dirty lines
+               back (up to 288 MB on this part) as its own reads evict them -- that figure
+               is reported beside it as latency_us.cold_after_write_flush_median.
   ms_per_step  wall clock of exactly --steps back-to-back calls / steps (warm caches,
                launch overhead included), after --warmup untimed calls.  Before those the
                device is kept busy with the same call for 200 ms (`device_warmup_ms` in the
@@ -273,14 +276,26 @@ def main():
 
     # ---- cold-cache latency per call (events on the launch stream, flush before every call)
     flush = torch.empty(1 << 28, dtype=torch.int32, device=device)     # 1 GiB
+
+    def flush_caches(clean=True):
+        flush.zero_()          # evicts the pool from L2 and the Infinity Cache ...
+        if clean:
+            flush.sum()        # ... and reading the buffer back leaves clean lines behind
     reps = COLD_CALLS
     cold, warm = [], []
     for _ in range(reps):
-        flush.zero_()
+        flush_caches()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(); step(); e1.record()
         e1.synchronize()
         cold.append(e0.elapsed_time(e1) * 1e3)
+    cold_dirty = []
+    for _ in range(max(30, reps // 4)):
+        flush_caches(clean=False)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(); step(); e1.record()
+        e1.synchronize()
+        cold_dirty.append(e0.elapsed_time(e1) * 1e3)
     for _ in range(reps):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(); step(); e1.record()
@@ -323,7 +338,7 @@ def main():
         ml = torch.empty((prob["batch"] * nsplit, prob["hq"]), dtype=torch.float32, device=device)
         ts = []
         for i in range(13):
-            flush.zero_()
+            flush_caches()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(); gathered_decode(inp.Q, k_cache, v_cache, lens, og, scale, 512, mo, ml); e1.record()
             e1.synchronize()
@@ -352,7 +367,7 @@ def main():
         om = torch.empty_like(inp.Q)
         ts = []
         for i in range(13):
-            flush.zero_()
+            flush_caches()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             fasttree_decode(inp.Q, inp.K_pool, inp.V_pool, om, *aux2, list(p2.TSQs), list(p2.TSKs), scale)
@@ -405,7 +420,8 @@ def main():
                    + f", {prob['hq']}q/{prob['hkv']}kv heads, head_dim 128, {prob['dtype']}, paged pool (page 1, shuffled), "
                    + f"{prob['batch']} requests", "planner_preset": args.preset,
                    "q_tiles": prob["q_tiles"], "vnodes": [int(x) for x in nums], "scratch_rows": int(rows)},
-        "latency_us": {"cold_median": cold_med, "cold_p20": cold_p20, "cold_p80": cold_p80, "warm_median": warm_med},
+        "latency_us": {"cold_median": cold_med, "cold_p20": cold_p20, "cold_p80": cold_p80,
+                       "cold_after_write_flush_median": statistics.median(cold_dirty), "warm_median": warm_med},
         "effective_kv": {"algorithmic_bytes": prob["algo_bytes"], "GBps": prob["algo_bytes"] / (cold_med * 1e-6) / 1e9,
                          "hbm_frac": prob["algo_bytes"] / (cold_med * 1e-6) / 1e9 / HBM_PEAK_GBS,
                          "algorithmic_gflop": prob["algo_flops"] / 1e9},
