@@ -76,6 +76,24 @@ def test_sweep_table_is_normalised_to_the_best_engine(tmp_path):
     assert "FAILED" in path.read_text().split("\n")[2]
 
 
+def test_plot_script_reads_the_sweep_table_and_draws_it(tmp_path):
+    """plot_norm_perf.py takes the table run_benchmark.py writes: one row per case of the chosen
+    preset, every engine column present, and a picture comes out."""
+    import plot_norm_perf
+    rows = [dict(tree=f"1,{n} / 8,8", heads=h, preset=p, flash_attn=0.4, naive=0.2, deft=0.125, node_wise=0.2, no_greedy=0.1,
+                 fasttree=0.05, check=True, deft_check=True, max_abs=1e-4, mean_abs=1e-5)
+            for n in (2, 4) for h in ("16/1", "32/8") for p in ("reference", "mi355x")]
+    table = tmp_path / "r.md"
+    run_benchmark.write_table(rows, str(table))
+    got = plot_norm_perf.read_table(str(table), "mi355x")
+    assert len(got) == 4 and all(r["preset"] == "mi355x" for r in got)
+    assert all(column in got[0] for column, _, _ in plot_norm_perf.ENGINES)
+    assert float(got[0]["tree ms"]) == 0.05 and float(got[0]["DeFT schedule ms"]) == 0.125
+    out = tmp_path / "r.png"
+    assert plot_norm_perf.main(["--input", str(table), "--preset", "mi355x", "--output", str(out)]) == 0
+    assert out.stat().st_size > 10000
+
+
 def test_deft_schedule_partitions_the_flattened_tree():
     """kernel_bench/DeFT.py:14-55 by hand on a small tree: depth-first token order, subtrees of
     `subtree_len` tokens, a node cut wherever a subtree is full; and on the trees of the
