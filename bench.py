@@ -9,14 +9,16 @@ reference bench (kernel_bench/benchmark.py:88-127).
 
 Prints ONE JSON line on stdout:
   value        median latency of one decode call in microseconds, measured with events
-               on the launch stream, every call preceded by a cache flush: a 1 GiB buffer is
-               rewritten and then read, so neither L2 nor the 256 MB Infinity Cache holds the
-               pool (inputs are resident in HBM, not in cache) and the lines they hold
-               instead are clean; 200 such calls whatever --steps is.  The reference's timer
-               (triton.testing.do_bench, kernel_bench/benchmark.py:59) only rewrites its
-               flush buffer: the call after it also pays for writing the buffer's dirty lines
-               back (up to 288 MB on this part) as its own reads evict them -- that figure
-               is reported beside it as latency_us.cold_after_write_flush_median.
+               on the launch stream, every call preceded by a cache flush as the reference's
+               timer does it (triton.testing.do_bench, kernel_bench/benchmark.py:35,59): a
+               flush buffer is rewritten, here 1 GiB instead of 256 MB because this part has
+               256 MB of Infinity Cache; 200 such calls whatever --steps is.  `value_method`
+               in the line names the method ("cold_median_after_write_flush") and does not
+               change between builds.  The call after such a flush also pays for writing the
+               buffer's dirty lines back (up to 288 MB on this part) as its own reads evict
+               them; the same call after a flush that rewrites the buffer AND reads it back
+               (clean lines in the caches, the pool still not in them) is reported beside it
+               as latency_us.cold_clean_median.
   ms_per_step  wall clock of exactly --steps back-to-back calls / steps (warm caches,
                launch overhead included), after --warmup untimed calls.  Before those the
                device is kept busy with the same call for 200 ms (`device_warmup_ms` in the
@@ -45,6 +47,9 @@ for extra in ("fasttree-artifact_amd", "oracle", os.path.join("tests", "golden")
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 DEVICE_WARMUP_MS = 200.0       # untimed calls before the --warmup steps, until the device's clocks have settled
 COLD_CALLS = 200               # flush + call repetitions behind `value` (their median)
+# How `value` is taken; fixed, so that the figure compares across builds: the median over COLD_CALLS
+# calls, each after the flush buffer has been rewritten (and not read back), as do_bench does it.
+VALUE_METHOD = "cold_median_after_write_flush"
 MFMA_PEAK_TFLOPS = 2500.0      # dense fp16 / bf16
 
 WORKLOADS = {
@@ -284,18 +289,18 @@ def main():
     reps = COLD_CALLS
     cold, warm = [], []
     for _ in range(reps):
-        flush_caches()
+        flush_caches(clean=False)        # the reference's method: the flush buffer is rewritten, nothing else
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(); step(); e1.record()
         e1.synchronize()
         cold.append(e0.elapsed_time(e1) * 1e3)
-    cold_dirty = []
+    cold_clean = []
     for _ in range(max(30, reps // 4)):
-        flush_caches(clean=False)
+        flush_caches(clean=True)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(); step(); e1.record()
         e1.synchronize()
-        cold_dirty.append(e0.elapsed_time(e1) * 1e3)
+        cold_clean.append(e0.elapsed_time(e1) * 1e3)
     for _ in range(reps):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(); step(); e1.record()
@@ -338,7 +343,7 @@ def main():
         ml = torch.empty((prob["batch"] * nsplit, prob["hq"]), dtype=torch.float32, device=device)
         ts = []
         for i in range(13):
-            flush_caches()
+            flush_caches(clean=False)
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(); gathered_decode(inp.Q, k_cache, v_cache, lens, og, scale, 512, mo, ml); e1.record()
             e1.synchronize()
@@ -367,7 +372,7 @@ def main():
         om = torch.empty_like(inp.Q)
         ts = []
         for i in range(13):
-            flush_caches()
+            flush_caches(clean=False)
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             fasttree_decode(inp.Q, inp.K_pool, inp.V_pool, om, *aux2, list(p2.TSQs), list(p2.TSKs), scale)
@@ -403,6 +408,7 @@ def main():
     result = {
         "metric": "tree-attention decode latency",
         "value": cold_med if parity["passed"] else None,
+        "value_method": VALUE_METHOD,
         "unit": "us",
         "n_gpus": 1,
         "steps": args.steps,
@@ -421,7 +427,7 @@ def main():
                    + f"{prob['batch']} requests", "planner_preset": args.preset,
                    "q_tiles": prob["q_tiles"], "vnodes": [int(x) for x in nums], "scratch_rows": int(rows)},
         "latency_us": {"cold_median": cold_med, "cold_p20": cold_p20, "cold_p80": cold_p80,
-                       "cold_after_write_flush_median": statistics.median(cold_dirty), "warm_median": warm_med},
+                       "cold_clean_median": statistics.median(cold_clean), "warm_median": warm_med},
         "effective_kv": {"algorithmic_bytes": prob["algo_bytes"], "GBps": prob["algo_bytes"] / (cold_med * 1e-6) / 1e9,
                          "hbm_frac": prob["algo_bytes"] / (cold_med * 1e-6) / 1e9 / HBM_PEAK_GBS,
                          "algorithmic_gflop": prob["algo_flops"] / 1e9},

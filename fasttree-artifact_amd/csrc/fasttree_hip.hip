@@ -17,7 +17,7 @@
 
 #include <hip/hip_runtime.h>
 #include <algorithm>
-#include <mutex>
+#include <atomic>
 #include <stdint.h>
 
 #include "../../include/fasttree_hip.h"
@@ -1516,14 +1516,15 @@ template <typename E, int D, int NQB, bool SPLIT, bool GATHERED>
 int launch_stage1_inst(const Stage1Args& a, int hkv, hipStream_t stream) {
   const size_t lds = (size_t)kWavesPerBlock * TileGeom<D>::kBytes;
   auto kern = stage1_kernel<E, D, NQB, SPLIT, GATHERED>;
-  static bool configured_on[kMaxDevices] = {};  // raising the dynamic LDS limit is idempotent
-  bool& configured = configured_on[current_device()];
-  if (!configured) {
+  // (raising the dynamic LDS limit is idempotent: two threads that both find the flag clear both raise it)
+  static std::atomic<bool> configured_on[kMaxDevices];
+  std::atomic<bool>& configured = configured_on[current_device()];
+  if (!configured.load(std::memory_order_acquire)) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
       (void)hipGetLastError();
       return FT_ERR_LAUNCH;
     }
-    configured = true;
+    configured.store(true, std::memory_order_release);
   }
   const unsigned gx = SPLIT ? (unsigned)a.vnode_count : (unsigned)((a.vnode_count + kWavesPerBlock - 1) / kWavesPerBlock);
   hipLaunchKernelGGL(kern, dim3(gx, (unsigned)hkv, 1), dim3(kBlock, 1, 1), lds, stream, a);
@@ -1535,16 +1536,20 @@ int launch_stage1_inst(const Stage1Args& a, int hkv, hipStream_t stream) {
 // waves would each walk a long run alone, one memory round trip per tile; with the slots nearly
 // full the runs are limited by memory bandwidth already and sharing only adds barriers.
 inline int wave_slots() {
-  static int slots = 0;
-  if (slots == 0) {
+  // per device; threads that race on the first call compute and store the same value
+  static std::atomic<int> slots_on[kMaxDevices];
+  std::atomic<int>& slots = slots_on[current_device()];
+  int n = slots.load(std::memory_order_relaxed);
+  if (n == 0) {
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
       (void)hipGetLastError();
       cus = 256;
     }
-    slots = cus * kWaveSlotsPerCu;
+    n = cus * kWaveSlotsPerCu;
+    slots.store(n, std::memory_order_relaxed);
   }
-  return slots;
+  return n;
 }
 inline int narrow_share_for(int64_t items, int head_dim) {
   const int slots = head_dim > 128 ? wave_slots() / 2 : wave_slots();   // (one block per compute unit at 512-byte rows)
@@ -1559,14 +1564,15 @@ int launch_stage1_fused(const Stage1Args& a0, hipStream_t stream) {
   constexpr size_t kNarrowLds = (size_t)kWideWaves * NarrowGeom<D>::kLds;
   constexpr size_t lds = kWideLds > kNarrowLds ? kWideLds : kNarrowLds;
   auto kern = stage1_fused_kernel<E, D, GATHERED>;
-  static bool configured_on[kMaxDevices] = {};  // raising the dynamic LDS limit is idempotent
-  bool& configured = configured_on[current_device()];
-  if (!configured) {
+  // (raising the dynamic LDS limit is idempotent: two threads that both find the flag clear both raise it)
+  static std::atomic<bool> configured_on[kMaxDevices];
+  std::atomic<bool>& configured = configured_on[current_device()];
+  if (!configured.load(std::memory_order_acquire)) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
       (void)hipGetLastError();
       return FT_ERR_LAUNCH;
     }
-    configured = true;
+    configured.store(true, std::memory_order_release);
   }
   Stage1Args a = a0;
   const int64_t narrow_items = (int64_t)(a.narrow_count - a.narrow_in_programs) * a.hkv;  // those of the trailing blocks
@@ -1592,15 +1598,16 @@ int launch_stage1_narrow(const Stage1Args& a0, hipStream_t stream) {
   a.narrow_share = narrow_share_for(blocks, D);
   auto kern = stage1_narrow_kernel<E, D, GATHERED>;
   const size_t lds = (size_t)a.narrow_share * NarrowGeom<D>::kLds;
-  static bool configured_on[kMaxDevices] = {};  // raising the dynamic LDS limit is idempotent
-  bool& configured = configured_on[current_device()];
-  if (!configured) {
+  // (raising the dynamic LDS limit is idempotent: two threads that both find the flag clear both raise it)
+  static std::atomic<bool> configured_on[kMaxDevices];
+  std::atomic<bool>& configured = configured_on[current_device()];
+  if (!configured.load(std::memory_order_acquire)) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             kWideWaves * NarrowGeom<D>::kLds) != hipSuccess) {
       (void)hipGetLastError();
       return FT_ERR_LAUNCH;
     }
-    configured = true;
+    configured.store(true, std::memory_order_release);
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)blocks, 1, 1), dim3(kWave * a.narrow_share, 1, 1), lds, stream, a);
   return hipGetLastError() == hipSuccess ? FT_OK : FT_ERR_LAUNCH;
@@ -1688,29 +1695,31 @@ static __device__ __align__(256) unsigned char scratch[FT_STATIC_SCRATCH_BYTES];
 
 static int static_scratch_of_current_device(char** out) {
   constexpr int kMaxDevices = 64;
-  static std::mutex guard;
-  static char* address[kMaxDevices] = {};
+  // No lock: the lookup gives every thread the same address for a device, so threads that race on
+  // a device's first call store the same pointer, and later calls are one atomic load.
+  static std::atomic<char*> address[kMaxDevices];
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
     (void)hipGetLastError();
     return FT_ERR_LAUNCH;
   }
-  std::lock_guard<std::mutex> lock(guard);
-  if (!address[dev]) {
-    char* ptr = nullptr;
+  char* ptr = address[dev].load(std::memory_order_acquire);
+  if (!ptr) {
     if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
       (void)hipGetLastError();
       return FT_ERR_LAUNCH;
     }
-    address[dev] = ptr;
+    address[dev].store(ptr, std::memory_order_release);
   }
-  *out = address[dev];
+  *out = ptr;
   return FT_OK;
 }
 
 extern "C" {
 
 const char* ft_version(void) { return "fasttree_hip 0.1 (gfx950)"; }
+
+int64_t ft_static_scratch_bytes(void) { return (int64_t)FT_STATIC_SCRATCH_BYTES; }
 
 const char* ft_error_string(int code) {
   switch (code) {

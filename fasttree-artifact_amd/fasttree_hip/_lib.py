@@ -24,6 +24,7 @@ _P = c_void_p
 SIGNATURES = {
     "ft_version": (c_char_p, []),
     "ft_error_string": (c_char_p, [c_int]),
+    "ft_static_scratch_bytes": (c_int64, []),
     "ft_stage1": (c_int, [_P, _P, _P] + _I64x6 + [_P] * 6 + [c_int] * 7 + [c_float]
                   + [_P, c_int64, c_int64, _P, c_int64, c_int, _P]),
     "ft_stage1_phases": (c_int, [_P, _P, _P] + _I64x6 + [_P] * 6 + [_P, c_int64, c_int64, _P, c_int64] + [_P] * 4

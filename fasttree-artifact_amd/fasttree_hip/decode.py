@@ -111,7 +111,7 @@ def fasttree_decode_static(q, k_buffer, v_buffer, o, vnode_to_kv_entries, vnode_
 
     Takes the lists of ``fasttree_preparation(launch_order=True)`` (``phase_node_nums`` carries
     the program table when there are wide vnodes).  Raises ``FastTreeLibraryError`` when the scratch rows
-    do not fit the library's array (128 MiB per device).  Calls that overlap on one device race
+    do not fit the library's array (``ft_static_scratch_bytes()``, 64 MiB per device as built).  Calls that overlap on one device race
     on that array."""
     assert q.shape[-1] == k_buffer.shape[-1]
     _need_gpu(q, k_buffer, v_buffer, o, vnode_to_kv_entries)

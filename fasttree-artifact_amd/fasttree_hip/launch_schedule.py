@@ -340,7 +340,9 @@ def _block_programs(runs, batch_size, group, num_kv_heads, *,
     wide_runs, narrow = [], []    # narrow: (kv_off, kv_len, requests) per planner chunk
     for start, lens, reqs in runs:
         rows = len(reqs) * group
-        if rows <= NARROW_ROWS:
+        # (a run without tokens has no tile steps to schedule: it goes with the narrow vnodes, whose
+        # waves write its empty partial results)
+        if rows <= NARROW_ROWS or sum(lens) == 0:
             off = start
             for length in lens:
                 narrow.append((off, length, reqs))

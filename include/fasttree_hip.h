@@ -167,17 +167,25 @@ int ft_decode_programs(const void* q, const void* k, const void* v, void* o,
  * allocates and frees nothing on host-visible APIs: no hipMalloc, no hipFree, no library routine
  * that allocates.
  *
- * num_rows is the number of scratch rows the lists refer to (the length of vnode_to_q_entries).
- * The array holds FT_STATIC_SCRATCH_BYTES on every device the library is used on, for the life
- * of the process; a call needs num_rows * num_qo_heads * head_dim * 4 bytes, rounded up to 256,
+ * num_rows is the number of scratch rows the lists refer to (the length of vnode_to_q_entries);
+ * it is trusted like the lists themselves: every vnode's q_off + q_len and every entry of
+ * req_to_vnode_entries must lie below it, or the first launch writes outside the part of the
+ * array that was checked against the capacity.
+ * The array holds FT_STATIC_SCRATCH_BYTES (64 MiB unless the library was built with another
+ * -DFT_STATIC_SCRATCH_BYTES=...) on every device of every process that loads the library, used or
+ * not, for the life of the process; a call needs num_rows * num_qo_heads * head_dim * 4 bytes, rounded up to 256,
  * plus num_rows * num_qo_heads * 4, and returns FT_ERR_SCRATCH when that is more.  The first
  * call on a device looks up the array's address on that device (make it before a capture
- * starts); later calls on that device only launch the two kernels.  All calls on one device
+ * starts); later calls on that device only launch the two kernels and take no lock.  All calls on one device
  * share the array: calls that overlap in time on one device (two streams, two threads) race on
  * it, and its contents are only meaningful between the two launches of one call.  Nothing in it
  * needs clearing: the first launch writes every row the second one reads.
  */
-#define FT_STATIC_SCRATCH_BYTES (128u << 20)
+#ifndef FT_STATIC_SCRATCH_BYTES
+#define FT_STATIC_SCRATCH_BYTES (64u << 20)
+#endif
+/* The capacity the loaded library was built with. */
+int64_t ft_static_scratch_bytes(void);
 int ft_decode_static(const void* q, const void* k, const void* v, void* o,
                      int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
                      int64_t oo0, int64_t oo1,

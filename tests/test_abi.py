@@ -22,7 +22,7 @@ def declared_symbols():
 def test_header_symbols_are_exported():
     names = declared_symbols()
     assert names == ["ft_decode", "ft_decode_programs", "ft_decode_static", "ft_error_string", "ft_gathered_decode", "ft_stage1",
-                     "ft_stage1_phases", "ft_stage1_programs", "ft_stage2", "ft_store_kv", "ft_version"]
+                     "ft_stage1_phases", "ft_stage1_programs", "ft_stage2", "ft_static_scratch_bytes", "ft_store_kv", "ft_version"]
     lib = ctypes.CDLL(_lib.LIB_PATH)
     for name in names:
         assert hasattr(lib, name), name
@@ -36,6 +36,7 @@ def test_version_and_error_strings():
     for code in range(-7, 0):
         assert lib.ft_error_string(code) not in (b"ok", b"unknown error")
     assert lib.ft_error_string(-99) == b"unknown error"
+    assert lib.ft_static_scratch_bytes() == 64 << 20
 
 
 def test_argument_checks_return_codes_without_touching_a_device():

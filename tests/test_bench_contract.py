@@ -34,3 +34,17 @@ def test_profiles_name_the_command_that_made_them():
 def test_more_than_one_gpu_is_refused():
     out = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert out.returncode == 2 and "ONE GPU" in out.stderr
+
+
+def test_value_is_the_cold_median_after_a_write_flush():
+    """`value` keeps one definition across builds: the median over the cold calls, each timed after
+    the flush buffer was rewritten and not read back (the reference's do_bench method,
+    kernel_bench/benchmark.py:35,59); the figure after a flush that leaves clean lines is a side
+    figure under latency_us."""
+    import bench
+    assert bench.VALUE_METHOD == "cold_median_after_write_flush"
+    text = open(os.path.join(ROOT, "bench.py")).read()
+    body = text[text.index("cold, warm = [], []"):text.index("cold_clean = []")]
+    assert "flush_caches(clean=False)" in body and "flush_caches(clean=True)" not in body and "flush_caches()" not in body
+    assert '"value": cold_med if parity["passed"] else None' in text and '"value_method": VALUE_METHOD' in text
+    assert '"cold_clean_median"' in text

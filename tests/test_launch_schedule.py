@@ -209,3 +209,25 @@ def test_preparation_in_launch_order_carries_the_programs():
         assert torch.equal(a, b)
     assert torch.equal(outs[0][11].prog_table, outs[1][11].prog_table)
     assert outs[1][11].prog_table.data_ptr() == buffers.prog_table.data_ptr()
+
+
+@pytest.mark.parametrize("kw", [dict(), dict(recut=True), dict(recut=True, layout="packed"), dict(recut=False)])
+def test_a_shared_run_without_tokens_is_scheduled(kw):
+    """A node of zero tokens shared by many requests (more than 16 query rows: a wide run with no
+    tile steps) is arranged like any other: it gets scratch rows, which the kernels fill with empty
+    partial results, and no program is built from nothing."""
+    reqs = 40
+    # vnode 0: the empty shared root; vnode 1: a shared run of 300 tokens; then one leaf per request
+    kv_offs = [0, 0] + [300 + 20 * r for r in range(reqs)]
+    kv_lens = [0, 300] + [20] * reqs
+    q_offs = [0, reqs] + [2 * reqs + r for r in range(reqs)]
+    q_lens = [reqs, reqs] + [1] * reqs
+    q_entries = list(range(reqs)) * 2 + list(range(reqs))
+    sched = block_programs(kv_offs, kv_lens, q_offs, q_lens, q_entries, reqs, 4, 8, **kw)
+    seen = _attended(sched.kv_offs, sched.kv_lens, sched.q_offs, sched.q_lens, sched.q_entries,
+                     sched.req_entries, sched.req_offs, sched.req_lens, reqs)
+    for r in range(reqs):
+        assert seen[r] == sorted(list(range(300)) + list(range(300 + 20 * r, 320 + 20 * r)))
+    # only the empty root everywhere: nothing to cut, nothing to fail on
+    alone = block_programs([0], [0], [0], [reqs], list(range(reqs)), reqs, 4, 8, **kw)
+    assert alone.num_rows == reqs and int(alone.kv_lens.sum()) == 0
