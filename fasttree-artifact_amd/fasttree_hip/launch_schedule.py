@@ -58,8 +58,12 @@ import numpy as np
 
 #: Query rows one block of the first-stage kernel serves per pass (4 waves x 32 rows).
 BLOCK_ROWS = 128
-#: Blocks of the first-stage kernel an MI355X runs at a time (two per compute unit).
-BLOCK_SLOTS = 512
+#: Blocks and waves of the first-stage kernel one compute unit holds at a time (72 KB of LDS and
+#: 238 registers per block of four waves).
+BLOCKS_PER_CU = 2
+WAVES_PER_CU = 8
+#: Compute units assumed when no device can be asked (an MI355X has 256).
+DEFAULT_COMPUTE_UNITS = 256
 #: KV tokens of one tile step.
 TILE_TOKENS = 32
 #: Start-up and wind-down of one vnode inside a program, in tile steps (three dependent memory
@@ -73,14 +77,13 @@ NARROW_STEP_TILES = 0.85
 #: and of one that does not (measured on the 3-level tree of the headline benchmark).
 TILE_US_SHARED = 1.19
 TILE_US_ALONE = 0.95
-#: Bytes per microsecond the narrow vnodes stream at most (rows of 2 * head_dim bytes at random slots).
+#: Bytes per microsecond the narrow vnodes stream at most on DEFAULT_COMPUTE_UNITS units (rows of
+#: 2 * head_dim bytes at random slots); taken to scale with the number of units.
 NARROW_BYTES_PER_US = 5.6e6
 #: A tile step of a piece of at most 64 query rows, relative to one of a full block.  The block's
 #: waves then split the tokens of a super tile, but the super tile is loaded all the same: fitted on
 #: the programs of an irregular tree of 500 requests, 1.21 against 1.44 us per tile step.
 LIGHT_TILE_WEIGHT = 0.85
-#: Waves the machine holds (narrow vnodes in flight).
-WAVE_SLOTS = 2048
 #: Waves of a block (each serves one narrow vnode at a time).
 BLOCK_WAVES = 4
 #: A launch is cut into equal programs only if every program gets at least this much work
@@ -144,8 +147,9 @@ class LaunchSchedule:
     prog_table: np.ndarray       # (num_programs, 4); see LaunchPhases
     narrow_in_programs: int
     program_tiles: np.ndarray    # modelled work of every program (for tests and reports)
-    block_slots: int = BLOCK_SLOTS
+    block_slots: int = BLOCKS_PER_CU * DEFAULT_COMPUTE_UNITS
     modelled_us: float = 0.0     # modelled duration of the launch
+    num_cus: int = DEFAULT_COMPUTE_UNITS   # compute units the launch was laid out for
 
     @property
     def num_rows(self) -> int:
@@ -154,6 +158,29 @@ class LaunchSchedule:
     @property
     def num_programs(self) -> int:
         return int(self.prog_table.shape[0])
+
+
+_CUS_OF_DEVICE = {}
+
+
+def compute_units(device=None) -> int:
+    """Compute units of ``device`` (a torch device, an index or None = the current one), as the
+    runtime reports them (``multi_processor_count``, the attribute the kernels' launcher reads as
+    well); :data:`DEFAULT_COMPUTE_UNITS` where no device is visible."""
+    try:
+        import torch
+
+        if not torch.cuda.is_available():
+            return DEFAULT_COMPUTE_UNITS
+        dev = torch.device(device) if device is not None else torch.device("cuda", torch.cuda.current_device())
+        if dev.type != "cuda":
+            return DEFAULT_COMPUTE_UNITS
+        index = dev.index if dev.index is not None else torch.cuda.current_device()
+        if index not in _CUS_OF_DEVICE:
+            _CUS_OF_DEVICE[index] = int(torch.cuda.get_device_properties(index).multi_processor_count)
+        return _CUS_OF_DEVICE[index]
+    except Exception:
+        return DEFAULT_COMPUTE_UNITS
 
 
 def _tile_weight(rows: int) -> float:
@@ -232,12 +259,15 @@ def _runs_of(kv_offs, kv_lens, q_offs, q_lens, q_entries):
 
 def block_programs(kv_offs, kv_lens, q_offs, q_lens, q_entries, batch_size, group, num_kv_heads, *,
                    block_rows=BLOCK_ROWS, block_slots=None, recut=None, embed=False, head_dim=128,
-                   layout=None, cuts=None) -> LaunchSchedule:
+                   layout=None, cuts=None, num_cus=None) -> LaunchSchedule:
     """The planner's lists arranged as block programs (see the module docstring).
 
     ``layout`` forces "packed" or "resident" programs (None: by modelled duration); ``cuts``
     forces how packed programs are made, "sequential" (filled one after the other) or "dealt"
     (equal pieces dealt to the least loaded program); both are for experiments and tests.
+
+    ``num_cus`` is the number of compute units the launch is laid out for (None: those of the
+    current device, :func:`compute_units`); the block and wave slots follow from it.
 
     With ``block_slots=None`` the launch is laid out twice, for programs on every block slot of
     the machine (two per compute unit: the narrow vnodes then wait for the programs to end) and
@@ -248,14 +278,15 @@ def block_programs(kv_offs, kv_lens, q_offs, q_lens, q_entries, batch_size, grou
     kv_offs, kv_lens, q_offs, q_lens = (np.asarray(x, dtype=np.int64) for x in (kv_offs, kv_lens, q_offs, q_lens))
     q_entries = np.asarray(q_entries, dtype=np.int64)
     runs = _runs_of(kv_offs, kv_lens, q_offs, q_lens, q_entries)
+    cus = max(1, int(num_cus)) if num_cus else compute_units()
     if block_slots is None:
         # (at head_dim 256 a compute unit holds one block of the kernel: 512-byte rows, 136 KB of LDS)
-        layouts = (BLOCK_SLOTS, BLOCK_SLOTS // 2) if head_dim <= 128 else (BLOCK_SLOTS // 2,)
-        both = [_block_programs(runs, batch_size, group, num_kv_heads,
+        layouts = (BLOCKS_PER_CU * cus, cus) if head_dim <= 128 else (cus,)
+        both = [_block_programs(runs, batch_size, group, num_kv_heads, num_cus=cus,
                                 block_rows=block_rows, block_slots=slots, recut=recut, embed=embed, head_dim=head_dim, layout=layout, cuts=cuts)
                 for slots in layouts]
         return min(both, key=lambda layout: layout[0])[1]()     # (only the chosen layout's lists are built)
-    return _block_programs(runs, batch_size, group, num_kv_heads,
+    return _block_programs(runs, batch_size, group, num_kv_heads, num_cus=cus,
                            block_rows=block_rows, block_slots=block_slots, recut=recut, embed=embed, head_dim=head_dim,
                            layout=layout, cuts=cuts)[1]()
 
@@ -318,7 +349,7 @@ def _resident_pieces(items, per_round, tiles, first_row):
 
 
 def _block_programs(runs, batch_size, group, num_kv_heads, *,
-                    block_rows, block_slots, recut, embed, head_dim, layout=None, cuts=None):
+                    block_rows, block_slots, recut, embed, head_dim, layout=None, cuts=None, num_cus=DEFAULT_COMPUTE_UNITS):
     """One layout of :func:`block_programs`, for ``block_slots`` programs at a time: its
     modelled duration and a function that builds its :class:`LaunchSchedule`.
 
@@ -334,6 +365,8 @@ def _block_programs(runs, batch_size, group, num_kv_heads, *,
     """
     group = max(1, int(group))
     heads = max(1, int(num_kv_heads))
+    machine_slots = BLOCKS_PER_CU * int(num_cus)      # blocks of the kernel the device holds at a time
+    wave_slots = WAVES_PER_CU * int(num_cus)          # waves (narrow vnodes in flight)
     cap = max(1, int(block_rows) // group)            # requests per row chunk
     per_round = max(1, int(block_slots) // heads)     # programs per round and head
 
@@ -455,7 +488,7 @@ def _block_programs(runs, batch_size, group, num_kv_heads, *,
             if cuts == "dealt" or d_max <= DEALT_MARGIN * max(load for _, load in filled):
                 pieces, programs = d_pieces, d_programs
         if layout != "packed":
-            resident = _resident_pieces(items, per_round, tiles, max(1, (BLOCK_SLOTS // 2) // heads))
+            resident = _resident_pieces(items, per_round, tiles, max(1, (machine_slots // 2) // heads))
     elif items:
         # The planner's chunks as they are, one vnode per program, longest first.  While the
         # launch would leave half of the machine idle, row chunks are halved (down to 64 rows):
@@ -508,7 +541,7 @@ def _block_programs(runs, batch_size, group, num_kv_heads, *,
         narrow = embedded + [v for v in narrow if id(v) not in taken]
 
         # ---- modelled duration of the launch (microseconds)
-        shared = len(programs) * heads > BLOCK_SLOTS // 2          # two program blocks on some compute unit
+        shared = len(programs) * heads > machine_slots // 2        # two program blocks on some compute unit
         tile_us = TILE_US_SHARED if shared else TILE_US_ALONE
         if programs:
             waves_of_blocks = max(1.0, len(programs) * heads / float(block_slots))
@@ -520,25 +553,25 @@ def _block_programs(runs, batch_size, group, num_kv_heads, *,
         if trailing:
             item_us = [narrow_work(v) * TILE_US_SHARED for v in trailing]
             narrow_bytes = sum(v[1] for v in trailing) * heads * 4 * head_dim
-            slots_for_narrow = WAVE_SLOTS if shared or not programs else WAVE_SLOTS // 2
+            slots_for_narrow = wave_slots if shared or not programs else wave_slots // 2
 
             def narrow_us(wave_slots):
-                return max(sum(item_us) * heads / wave_slots, max(item_us), narrow_bytes / NARROW_BYTES_PER_US)
+                return max(sum(item_us) * heads / wave_slots, max(item_us), narrow_bytes / (NARROW_BYTES_PER_US * num_cus / DEFAULT_COMPUTE_UNITS))
 
             if overlap:
                 # unequal programs end one after the other and the trailing blocks take their slots
                 # while the longest still run: the launch lasts as long as its longest program, or
                 # as long as all the work takes on all the slots
-                first_row = max(1, (BLOCK_SLOTS // 2) // heads)      # programs that are the older block of their unit
+                first_row = max(1, (machine_slots // 2) // heads)    # programs that are the older block of their unit
                 if shared:
                     longest_us = max(t * TILE_US_OLDER * (YOUNGER_BLOCK_SLOWDOWN if i >= first_row else 1.0)
                                      for i, t in enumerate(program_tiles))
                 else:
                     longest_us = max(program_tiles) * tile_us
                 modelled = max(longest_us,
-                               sum(program_tiles) * heads / float(block_slots) * tile_us + narrow_us(WAVE_SLOTS))
+                               sum(program_tiles) * heads / float(block_slots) * tile_us + narrow_us(wave_slots))
             else:
-                modelled = wide_us + narrow_us(WAVE_SLOTS) if shared else max(wide_us, narrow_us(slots_for_narrow))
+                modelled = wide_us + narrow_us(wave_slots) if shared else max(wide_us, narrow_us(slots_for_narrow))
         else:
             modelled = wide_us
 
@@ -584,7 +617,7 @@ def _block_programs(runs, batch_size, group, num_kv_heads, *,
                 phase_node_nums=[n_wide, len(new_kv_offs) - n_wide], phase_node_offsets=[0, n_wide],
                 prog_table=i32(prog_table).reshape(-1, 4), narrow_in_programs=narrow_first,
                 program_tiles=np.asarray(program_tiles, dtype=np.float64), block_slots=int(block_slots),
-                modelled_us=float(modelled),
+                modelled_us=float(modelled), num_cus=int(num_cus),
             )
 
         return float(modelled), build

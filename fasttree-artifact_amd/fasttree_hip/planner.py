@@ -479,6 +479,7 @@ def fasttree_preparation(
     kv_slot_map=None,
     launch_order=False,
     buffers=None,
+    num_cus=None,
 ):
     """Drop-in for kernel_bench/fasttree.py:99-296: plan on the host, then place the nine
     int32 index arrays and the two fp32 partial-result buffers on ``device``.
@@ -495,7 +496,8 @@ def fasttree_preparation(
     ``launch_order=True`` the lists come back arranged for an MI355X instead
     (:func:`launch_schedule.block_programs`: the same computation as block programs,
     with scratch rows and per-request lists of its own); ``phase_node_nums`` is then a list that
-    also carries the program table, which ``fasttree_decode`` picks up.
+    also carries the program table, which ``fasttree_decode`` picks up; the programs are laid out
+    for ``num_cus`` compute units (None: those ``device`` reports, 256 where it is not a GPU).
     """
     import torch
 
@@ -525,7 +527,10 @@ def fasttree_preparation(
     phase_nums, phase_offs = list(plan.phase_node_nums), list(plan.phase_node_offsets)
     if launch_order:
         group = max(1, num_qo_heads // num_kv_heads)
-        sched = block_programs(*vnodes, q_entries, batch_size, group, num_kv_heads, head_dim=head_dim)
+        if num_cus is None:
+            from .launch_schedule import compute_units
+            num_cus = compute_units(device)
+        sched = block_programs(*vnodes, q_entries, batch_size, group, num_kv_heads, head_dim=head_dim, num_cus=num_cus)
         vnodes = (sched.kv_offs, sched.kv_lens, sched.q_offs, sched.q_lens)
         q_entries = sched.q_entries
         per_request = (sched.req_entries, sched.req_offs, sched.req_lens)

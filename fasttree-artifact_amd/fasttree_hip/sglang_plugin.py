@@ -338,8 +338,9 @@ def prepare_for_fasttree_meta(batch, fasttree_metadata: FastTreeMetadata):
         # the same computation as block programs: long shared runs (a system prompt
         # under a large batch) cut where the machine is full instead of at the KV split
         tail_ends = [lists[0][v] + lists[1][v] for v in meta.req_last_vnodes]
+        from .launch_schedule import compute_units
         sched = block_programs(*lists, q_entries, len(batch.reqs), meta.kv_group_num, meta.num_kv_heads,
-                               head_dim=meta.head_dim)
+                               head_dim=meta.head_dim, num_cus=compute_units(meta.device))
         lists = [sched.kv_offs, sched.kv_lens, sched.q_offs, sched.q_lens]      # (int32 arrays, uploaded as they are)
         q_entries = sched.q_entries
         req_entries = sched.req_entries[: sched.num_rows]

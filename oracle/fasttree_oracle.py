@@ -20,6 +20,11 @@ checkout):
 * ``stage2_arith``               _fwd_fasttree_decoding_stage2, fasttree.py:498-546: tiles of
                                  4 partials, running max / sum, missing entries count as
                                  lse = -inf, o = 0; result rounded to the output type.
+* ``decode_arith_for_requests``  both of the above for a few requests of a given plan (every
+                                 scratch row of a sampled request as a one-request vnode over
+                                 the same KV slice): the like-for-like reference of the
+                                 bfloat16 cases, where the storage type is coarser than the
+                                 parity bar.
 * ``plan``                       cost model, greedy splitter, 3-pass adaptation and vnode
                                  emission, fasttree.py:30-96 and :111-262.
 * ``gathered_attention_torch``   the "no prefix sharing" formulation on the CPU with PyTorch
@@ -32,7 +37,8 @@ fixtures written by the reference planner (tests/golden/planner_goldens.json), p
 hand-derived known answers; ``stage1_arith``/``stage2_arith`` and ``dense_attention``
 against outputs of the reference's own kernels executed under Triton's CPU interpreter
 (tests/golden/kernel_*.npz), plus closed forms (single key, uniform keys, split
-invariance).  No function here is left unpinned.
+invariance); ``decode_arith_for_requests`` against the same kernel outputs for the requests it
+is given and against the whole-plan arithmetic.  No function here is left unpinned.
 """
 
 from __future__ import annotations
@@ -144,6 +150,43 @@ def fasttree_decode_arith(q, k_pool, v_pool, plan, kv_tile: int, sm_scale: float
     o = stage2_arith(plan.req_to_vnode_entries[:-n_pad], plan.req_to_vnode_offs, plan.req_to_vnode_lens,
                      mid_o, mid_lse, q.dtype)
     return o, mid_o, mid_lse
+
+
+def decode_arith_for_requests(q, k_pool, v_pool, lists, sample, kv_tile: int, sm_scale: float, remap=None):
+    """The two-stage arithmetic (stage1_arith, stage2_arith: P rounded to the storage type before
+    P.V, fp32 accumulation, the output rounded to the storage type; kernel_bench/fasttree.py:
+    384-413, 534-546) for the requests ``sample`` only, on a given plan: ``lists`` are the nine
+    index arrays of kernel_bench/fasttree.py:265-280 as numpy arrays (any vnode order).  Every
+    scratch row of a sampled request becomes a one-request vnode over the same KV slice, so the
+    cost is that of the sampled requests' own paths.  ``q`` holds the sampled requests only, in
+    order; ``remap`` translates pool slots when ``k_pool`` / ``v_pool`` hold only the rows the
+    sample needs.  Returns ``o [len(sample), Hq, D]`` in ``q.dtype``."""
+    kv_entries, kv_offs, kv_lens, q_entries, q_offs, q_lens, req_entries, req_offs, req_lens = lists
+    kv_entries = np.asarray(kv_entries).reshape(-1)
+    vnode_by_row = np.empty(len(q_entries), dtype=np.int64)
+    for v in range(len(q_offs)):
+        vnode_by_row[q_offs[v]: q_offs[v] + q_lens[v]] = v
+    new_entries, new_kv_offs, new_kv_lens, new_q = [], [], [], []
+    r_entries, r_offs, r_lens = [], [], []
+    for i, r in enumerate(sample):
+        rows = req_entries[req_offs[r]: req_offs[r] + req_lens[r]]
+        r_offs.append(len(new_q))
+        r_lens.append(len(rows))
+        for row in rows:
+            assert q_entries[row] == r, "a request's list names a scratch row of another request"
+            v = vnode_by_row[row]
+            slots = kv_entries[kv_offs[v]: kv_offs[v] + kv_lens[v]]
+            if remap is not None:
+                slots = [remap[int(s)] for s in slots]
+            new_kv_offs.append(len(new_entries))
+            new_kv_lens.append(len(slots))
+            new_entries.extend(int(s) for s in slots)
+            r_entries.append(len(new_q))
+            new_q.append(i)
+    n = len(new_q)
+    mid_o, mid_lse = stage1_arith(q, k_pool, v_pool, np.asarray(new_entries, dtype=np.int64), new_kv_offs,
+                                  new_kv_lens, new_q, list(range(n)), [1] * n, kv_tile, sm_scale, n)
+    return stage2_arith(r_entries, r_offs, r_lens, mid_o, mid_lse, q.dtype)
 
 
 def gathered_attention_torch(q, k_pool, v_pool, path_tokens, sm_scale, requests=None):

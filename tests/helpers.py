@@ -98,3 +98,35 @@ def plan_to_device(plan, hq, d, device):
         torch.full((rows, hq), float("nan"), dtype=torch.float32, device=device),
         list(plan.phase_node_nums), list(plan.phase_node_offsets),
     )
+
+
+
+def arith_reference(q, k_pool, v_pool, aux, sample, kv_tile, sm_scale, remap=None):
+    """The reference kernels' own arithmetic in the storage type, for the requests ``sample`` on the
+    very plan ``aux`` (see oracle.decode_arith_for_requests)."""
+    import fasttree_oracle as oracle
+
+    lists = [t.detach().cpu().numpy() for t in aux[:9]]
+    return oracle.decode_arith_for_requests(q, k_pool, v_pool, lists, sample, kv_tile, sm_scale, remap=remap)
+
+
+def assert_like_for_like(got, want, what="", strict=False):
+    """``got`` against the reference arithmetic evaluated in the same 16-bit type (``want``, from
+    :func:`arith_reference`): mean-abs at the plain bar; max-abs at the plain bar or, where one
+    unit in the last place of the expected value is coarser than the bar (bfloat16 values of
+    magnitude 0.5 and more: 2**-8 and up), at most that one unit -- the two results are then
+    neighbouring representable values.  ``strict`` holds every element to the plain bar."""
+    g = got.detach().cpu().to(torch.float64)
+    w = want.detach().cpu().to(torch.float64)
+    diff = (g - w).abs()
+    worst_max = float(diff.max())
+    worst_mean = float(diff.reshape(g.shape[0], -1).mean(dim=1).max())
+    allowed = torch.full_like(w, MAX_ABS_TOL)
+    if not strict:
+        mant_bits = 7 if want.dtype == torch.bfloat16 else 10
+        ulp = torch.exp2(torch.floor(torch.log2(w.abs().clamp_min(2.0 ** -126))) - mant_bits)
+        allowed = torch.maximum(allowed, ulp)
+    over = float((diff - allowed).max())
+    assert over <= 0 and worst_mean <= MEAN_ABS_TOL, (
+        f"{what}: like for like max-abs {worst_max:.3e} (over the allowance by {over:.3e}), mean-abs {worst_mean:.3e}")
+    return worst_max, worst_mean

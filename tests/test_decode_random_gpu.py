@@ -15,7 +15,7 @@ from cases import build_tree
 from fasttree_hip.decode import fasttree_decode, gathered_decode
 from fasttree_hip.inputs import gather_per_request, make_decode_inputs
 from fasttree_hip.planner import FastTreeParams, fasttree_preparation
-from helpers import assert_parity
+from helpers import arith_reference, assert_like_for_like, assert_parity
 
 pytestmark = pytest.mark.gpu
 
@@ -84,5 +84,11 @@ def test_random_tree_and_settings(seed, device):
     if c["dtype"] == torch.bfloat16:
         p_round = oracle.dense_attention(q_cpu[reqs], k_cpu, v_cpu.abs(), paths, scale) * 2.0 ** -9
         assert_parity(o[reqs], dense, f"random {seed}", out_dtype=torch.bfloat16, extra=p_round)
+        # like for like: the reference kernels' arithmetic in bfloat16 on the same plan (fasttree.py:391)
+        same_type = arith_reference(q_cpu[reqs], k_cpu, v_cpu, aux, reqs, 32, scale)
+        like = assert_like_for_like(o[reqs], same_type, f"random {seed}, like for like")
+        raw = (o[reqs].cpu().double() - dense).abs()
+        print(f"  bf16 random {seed}: vs bf16 arithmetic max-abs {like[0]:.2e} mean-abs {like[1]:.2e}; vs fp64 raw max-abs "
+              f"{float(raw.max()):.2e}", flush=True)
     else:
         assert_parity(o[reqs], dense.to(torch.float16), f"random {seed}")

@@ -231,3 +231,33 @@ def test_a_shared_run_without_tokens_is_scheduled(kw):
     # only the empty root everywhere: nothing to cut, nothing to fail on
     alone = block_programs([0], [0], [0], [reqs], list(range(reqs)), reqs, 4, 8, **kw)
     assert alone.num_rows == reqs and int(alone.kv_lens.sum()) == 0
+
+
+@pytest.mark.parametrize("num_cus", [128, 256, 304])
+@pytest.mark.parametrize("name", ["c3", "c5_seed0", "shape07_h32_8"])
+def test_layout_follows_the_number_of_compute_units(name, num_cus):
+    """The programs are laid out for the device's compute units, not for a fixed machine: on 128
+    units (a partitioned or smaller part) and on 304 (an MI300X) the same plan gives a schedule
+    with the same coverage whose programs of one round fit that machine's block slots -- two per
+    unit, or one per unit where that layout's modelled duration is the shorter."""
+    case = next(c for c in PLANNER_CASES if c["name"] == name)
+    plan, batch, group, s = _schedule(case, num_cus=num_cus)
+    assert s.num_cus == num_cus and s.block_slots in (num_cus, 2 * num_cus)
+    want = _attended(*_plan_lists(plan), plan.req_to_vnode_entries, plan.req_to_vnode_offs, plan.req_to_vnode_lens, batch)
+    got = _attended(s.kv_offs, s.kv_lens, s.q_offs, s.q_lens, s.q_entries, s.req_entries, s.req_offs, s.req_lens, batch)
+    assert got == want
+    heads = case["Hkv"]
+    rounds = max(1, int(np.ceil(s.program_tiles.sum() / ((s.block_slots // heads) * ls.MAX_PROGRAM_TILES)))) if s.num_programs else 1
+    assert s.num_programs <= max(1, s.block_slots // heads) * rounds or s.num_programs == s.phase_node_nums[0]
+
+
+def test_fewer_compute_units_mean_fewer_and_longer_programs():
+    case = next(c for c in PLANNER_CASES if c["name"] == "c3")
+    small = _schedule(case, num_cus=128, layout="packed")[3]
+    full = _schedule(case, num_cus=256, layout="packed")[3]
+    large = _schedule(case, num_cus=304, layout="packed")[3]
+    assert small.num_programs < full.num_programs <= large.num_programs
+    assert small.program_tiles.max() > full.program_tiles.max() >= large.program_tiles.max()
+    assert small.modelled_us > full.modelled_us >= large.modelled_us
+    # without a device to ask, the default machine is an MI355X's 256 units
+    assert ls.compute_units("cpu") == 256 == ls.DEFAULT_COMPUTE_UNITS

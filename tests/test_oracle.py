@@ -66,6 +66,30 @@ def test_two_stage_arithmetic_matches_reference_kernels(case):
 
 
 @pytest.mark.parametrize("case", KERNEL_CASES, ids=[c["name"] for c in KERNEL_CASES])
+def test_arithmetic_for_sampled_requests_matches_reference_kernels(case):
+    """decode_arith_for_requests (the two-stage arithmetic for a few requests of a plan, what the
+    bfloat16 GPU cases are compared with like for like) against what the reference's own kernels
+    wrote for those requests, and, where the whole plan is cheap enough to evaluate, against
+    fasttree_decode_arith on the whole plan: restricting a plan to some of its requests changes
+    nothing for them."""
+    tree, ptrs, batch, plan, q, k, v, gold = _kernel_case(case)
+    sm_scale = 1.0 / math.sqrt(case["D"])
+    kept = gold["requests"].tolist() if "requests" in gold else list(range(batch))
+    want = bits16_to_tensor(gold["o"], DTYPES[case["dtype"]])
+    picks = sorted(set(range(0, len(kept), max(1, len(kept) // 5))))        # positions within the fixture's requests
+    sample = [kept[i] for i in picks]
+    lists = [np.asarray(getattr(plan, name)) for name in ARRAYS[:9]]
+    o = oracle.decode_arith_for_requests(q[sample], k, v, lists, sample, case["TSKs"][0], sm_scale)
+    worst_max, worst_mean = per_request_errors(o, want[picks])
+    one_ulp = 2e-3 if case["dtype"] == "fp16" else 1.6e-2
+    assert worst_max <= one_ulp and worst_mean <= one_ulp / 20
+    if case["name"] != "k_c1" and not case.get("keep_every"):
+        full, _, _ = oracle.fasttree_decode_arith(q, k, v, plan, case["TSKs"][0], sm_scale)
+        assert torch.allclose(o.float(), full[sample].float(), rtol=0, atol=1e-3 if case["dtype"] == "fp16" else 8e-3)
+        assert (o.float() - full[sample].float()).abs().mean() <= 2e-5
+
+
+@pytest.mark.parametrize("case", KERNEL_CASES, ids=[c["name"] for c in KERNEL_CASES])
 def test_dense_identity_matches_reference_kernels(case):
     """Tree attention == dense soft-max attention of each request over its root path."""
     tree, ptrs, batch, plan, q, k, v, gold = _kernel_case(case)

@@ -546,3 +546,137 @@ def test_hook_replans_for_new_requests_and_every_few_forwards():
         gc.collect()
         batch.reqs = [Req([4], [])]               # ... and a new request is made, possibly at the same address
     assert calls.count("plan") == 54 and calls.count("step") == 4
+
+
+# ---- the loader, with stand-ins for the SGLang modules it patches
+def _install_sglang_stubs(monkeypatch, continue_steps=3):
+    """Modules with the names and the few members load_fasttree_plugin touches (SGLang v0.2.13:
+    RadixAttention, ModelTpServer, InputMetadata.from_schedule_batch, global_config); each records
+    what the patched versions hand on to it."""
+    import sys
+    import types
+
+    log = []
+
+    class RadixAttention:
+        def __init__(self, num_heads, head_dim, scaling, num_kv_heads, layer_id):
+            self.tp_q_head_num, self.qk_head_dim, self.v_head_dim = num_heads, head_dim, head_dim
+            self.scaling, self.layer_id, self.logit_cap = scaling, layer_id, -1
+
+        def decode_forward(self, q, k, v, input_metadata):
+            return "sglang decode"
+
+    class ModelTpServer:
+        def __init__(self, gpu_id, tp_rank, server_args, nccl_port, model_overide_args):
+            log.append(("server init", server_args.disable_cuda_graph))
+            self.gpu_id, self.tp_rank = gpu_id, tp_rank
+            self.model_config = Obj(num_attention_heads=32, num_key_value_heads=8, head_dim=128)
+
+        def forward_prefill_batch(self, batch):
+            log.append(("prefill", batch))
+            return "prefilled"
+
+        def forward_decode_batch(self, batch):
+            log.append(("decode", batch))
+            return "decoded"
+
+    class InputMetadata:
+        @classmethod
+        def from_schedule_batch(cls, model_runner, batch, forward_mode):
+            ret = cls()
+            ret.made_from = (model_runner, batch, forward_mode)
+            return ret
+
+    def module(name, **members):
+        mod = types.ModuleType(name)
+        mod.__dict__.update(members)
+        monkeypatch.setitem(sys.modules, name, mod)
+        return mod
+
+    module("sglang")
+    module("sglang.srt")
+    module("sglang.srt.layers")
+    module("sglang.srt.layers.radix_attention", RadixAttention=RadixAttention)
+    module("sglang.srt.managers")
+    module("sglang.srt.managers.tp_worker", ModelTpServer=ModelTpServer)
+    module("sglang.srt.model_executor")
+    module("sglang.srt.model_executor.forward_batch_info", InputMetadata=InputMetadata)
+    module("sglang.global_config", global_config=Obj(num_continue_decode_steps=continue_steps))
+    # (the reference's own plugin package must not be found: its loader would be used instead)
+    monkeypatch.setitem(sys.modules, "fasttree_sglang_plugin_v0_2_13", None)
+    return Obj(RadixAttention=RadixAttention, ModelTpServer=ModelTpServer, InputMetadata=InputMetadata, log=log)
+
+
+@pytest.mark.parametrize("annotate", [False, True])
+def test_loader_patches_the_three_sglang_classes(monkeypatch, annotate):
+    """load_fasttree_plugin without the reference's plugin package (plugin.py:190-238): every
+    RadixAttention instance gets the hook bound as its decode_forward, InputMetadata carries the
+    batch's metadata as .fasttree, ModelTpServer switches graphs off, creates the metadata from
+    its model config and, before every decode forward, plans (new requests, or the plan has served
+    num_continue_decode_steps forwards) or steps."""
+    import fasttree_hip.sglang_plugin as plugin
+
+    sg = _install_sglang_stubs(monkeypatch, continue_steps=3)
+    made = []
+
+    class Metadata:
+        def __init__(self, num_qo_heads, num_kv_heads, head_dim, device):
+            made.append((num_qo_heads, num_kv_heads, head_dim, str(device)))
+
+    planned = []
+    monkeypatch.setattr(plugin, "FastTreeMetadata", Metadata)
+    monkeypatch.setattr(plugin, "prepare_for_fasttree_meta", lambda batch, meta: planned.append(("plan", batch, meta)))
+    monkeypatch.setattr(plugin, "prepare_for_fasttree_step", lambda batch, meta: planned.append(("step", batch, meta)))
+    # the patched classes are this test's own stand-ins: nothing to restore but the module's two functions
+    plugin.load_fasttree_plugin(True, annotate)
+
+    layer = sg.RadixAttention(32, 128, 0.088, 8, layer_id=5)
+    assert layer.decode_forward.__func__ is plugin.decode_forward_fasttree and layer.decode_forward.__self__ is layer
+    other = sg.RadixAttention(32, 128, 0.088, 8, layer_id=6)
+    assert other.decode_forward.__self__ is other          # bound per instance, as plugin.py:58 does
+
+    meta = object()
+    batch = Obj(reqs=[Req([1], []), Req([2], [])], fasttree_metadata=meta)
+    im = sg.InputMetadata.from_schedule_batch("runner", batch, "DECODE")
+    assert im.fasttree is meta and im.made_from == ("runner", batch, "DECODE")
+    assert sg.InputMetadata.from_schedule_batch("runner", Obj(reqs=[]), "EXTEND").fasttree is None
+
+    args = Obj(disable_cuda_graph=False)
+    server = sg.ModelTpServer(1, 0, args, 28000, {})
+    assert args.disable_cuda_graph is True and sg.log[0] == ("server init", True)   # set before SGLang's own init runs
+    assert made == [(32, 8, 128, "cuda:1")]
+    assert isinstance(server.fasttree_metadata, Metadata)
+
+    assert [server.forward_decode_batch(batch) for _ in range(4)] == ["decoded"] * 4
+    assert [p[0] for p in planned] == ["plan", "step", "step", "plan"]
+    assert all(p[1] is batch and p[2] is server.fasttree_metadata for p in planned)
+    batch.reqs = batch.reqs[:1]                      # a request finished: other requests, a new plan
+    server.forward_decode_batch(batch)
+    assert planned[-1][0] == "plan"
+    assert [e[0] for e in sg.log].count("decode") == 5  # SGLang's own forward still runs, after the plan
+    assert server.forward_prefill_batch(batch) == "prefilled"
+    if annotate:
+        assert hasattr(sg.ModelTpServer.forward_prefill_batch, "__wrapped__")
+
+
+def test_loader_does_nothing_when_everything_is_off(monkeypatch, capsys):
+    import fasttree_hip.sglang_plugin as plugin
+
+    sg = _install_sglang_stubs(monkeypatch)
+    before = (sg.RadixAttention.__init__, sg.ModelTpServer.__init__, sg.ModelTpServer.forward_decode_batch)
+    plugin.load_fasttree_plugin(False, False)
+    assert "[Warning] FastTree plugin is not enabled" in capsys.readouterr().out        # plugin.py:235-237
+    assert before == (sg.RadixAttention.__init__, sg.ModelTpServer.__init__, sg.ModelTpServer.forward_decode_batch)
+    # the breakdown alone wraps SGLang's two forwards and leaves the attention path as it is
+    plugin.load_fasttree_plugin(False, True)
+    assert hasattr(sg.ModelTpServer.forward_decode_batch, "__wrapped__")
+    assert sg.RadixAttention(32, 128, 0.088, 8, 0).decode_forward(None, None, None, None) == "sglang decode"
+
+
+def test_loader_needs_sglang(monkeypatch):
+    import sys
+    import fasttree_hip.sglang_plugin as plugin
+    for name in ("fasttree_sglang_plugin_v0_2_13", "sglang", "sglang.srt.layers.radix_attention"):
+        monkeypatch.setitem(sys.modules, name, None)
+    with pytest.raises(ImportError):
+        plugin.load_fasttree_plugin(True, False)
