@@ -647,14 +647,20 @@ __device__ __forceinline__ u32x2 lds_read_tr8(unsigned addr) {
 // accumulators are rescaled rarely (in practice once, on a run's first tile).
 constexpr float kSlack = 8.f;
 
+// A tile step without a per-query mask (every row of the vnode attends every token of the run).
+struct NoMask {
+  __device__ __forceinline__ void operator()(f32x16&) const {}
+};
+
 // One 32-token step for the wave's 32 rows on the tile `off` bytes into the current buffer.
 // S^T = K Q^T: A = K rows (token lane%32, 8 dims per lane), B = Q; accumulator register j of a
 // lane is token 8*(j/4) + 4*(lane/32) + j%4.  Registers 8u .. 8u+7 are exactly the 8 k-slots a
 // lane feeds to the u-th P.V contraction, whose A operand (V^T) comes from two transposed LDS
-// reads of 4 consecutive tokens each.  valid < 32 only on a run's last, partial tile.
-template <typename E, int D>
+// reads of 4 consecutive tokens each.  valid < 32 only on a run's last, partial tile.  `mask`
+// is applied to the raw scores (it overwrites those of tokens the lane's row does not attend).
+template <typename E, int D, typename Mask = NoMask>
 __device__ __forceinline__ void tile_step32(const WideLane& la, unsigned off, int valid, float sc,
-                                            const u32x4 (&qf)[D / 16], WideState<D>& st) {
+                                            const u32x4 (&qf)[D / 16], WideState<D>& st, const Mask& mask = Mask()) {
   using W = WideGeom<D>;
   constexpr int KS = D / 16, DB = D / 32, NV = 2 * DB;
 
@@ -683,6 +689,7 @@ __device__ __forceinline__ void tile_step32(const WideLane& la, unsigned off, in
 #pragma unroll
     for (int j = 0; j < 16; ++j) s[j] = (8 * (j >> 2) + 4 * h + (j & 3) >= valid) ? -INFINITY : s[j];
   }
+  mask(s);
 
   // the V^T operands do not depend on the probabilities: request them now, so that they arrive
   // under the soft-max arithmetic (they take the registers the K operands just left); at
@@ -746,7 +753,8 @@ __device__ __forceinline__ void finish_state(WideState<D>& st) {
   st.l = xor32_sum(st.l);
 }
 
-template <int D>
+// (ROUND16: the normalised output is rounded to fp16 on its way to the fp32 scratch)
+template <int D, bool ROUND16 = false>
 __device__ __forceinline__ void write_partials32(const Stage1Args& a, const VnodeView& vn, int kvh, int row0,
                                                  const WideState<D>& st) {
   const int lane = threadIdx.x & 63;
@@ -761,8 +769,12 @@ __device__ __forceinline__ void write_partials32(const Stage1Args& a, const Vnod
   for (int db = 0; db < D / 32; ++db)
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
-      const f32x4 v = {st.o[db][4 * jj] * inv, st.o[db][4 * jj + 1] * inv, st.o[db][4 * jj + 2] * inv,
-                       st.o[db][4 * jj + 3] * inv};
+      f32x4 v = {st.o[db][4 * jj] * inv, st.o[db][4 * jj + 1] * inv, st.o[db][4 * jj + 2] * inv,
+                 st.o[db][4 * jj + 3] * inv};
+      if constexpr (ROUND16) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = (float)(_Float16)v[e];
+      }
       *reinterpret_cast<f32x4*>(dst + 32 * db + 8 * jj) = v;
     }
   if (h == 0) a.mid_lse[row * a.sl0 + head] = st.l > 0.f ? (__builtin_amdgcn_logf(st.l) + st.m) * kLn2 : -INFINITY;
@@ -1381,6 +1393,130 @@ __global__ void __launch_bounds__(kWideBlock, D > 128 ? 1 : 512 / kWideBlock) st
 }
 
 // ---------------------------------------------------------------------------------------
+// DeFT-Flatten's first stage (the comparison engine of the reference's benchmark,
+// kernel_bench/DeFT.py:194-340): one block per (subtree, kv head).  A subtree is a run of
+// consecutive tokens of the depth-first token order (128 in the benchmark) that may span
+// several tree nodes; its query set holds every request that attends any of its tokens, and a
+// 64-bit word per (group of mask_len requests, token) says which requests of the group attend the
+// token.  The block keeps up to 128 tokens of the subtree in LDS (the two super-tile buffers of
+// the wide kernel, same layout, same direct loads) and passes its query rows over them 128 at a
+// time, 32 per wave, with the scores of tokens a row does not attend set to a large negative
+// value before the soft-max (DeFT.py:283-306).  The partial output is rounded to fp16 on its
+// way to the fp32 scratch, as the reference kernel does (DeFT.py:391).
+// ---------------------------------------------------------------------------------------
+struct DeftArgs {
+  Stage1Args s;                    // tensors, strides, the six vnode lists (vnode = subtree), scale, scratch
+  const int64_t* causalmask;       // per subtree: [groups of mask_len requests][kv_len] words
+  const int32_t* causalmask_offset;
+  int mask_len;                    // requests per mask word: a power of two, at most 64
+  int num_subtrees;
+};
+
+constexpr int kDeftChunk = 2 * 64;       // tokens held in LDS at a time (both ring buffers)
+// Raw score of a token a row does not attend (the reference writes -1e6 over the scaled score,
+// DeFT.py:306).  Finite and moderate on purpose: a tile in which a row attends nothing makes this
+// value the row's soft-max reference, and the probabilities of that tile come out as exp2 of the
+// rounding error of (score * scale) -- about 1 for this magnitude, infinite for a huge one.  They
+// are garbage either way and are wiped out (factor exp2(-1e5) = 0) by the first attended token.
+constexpr float kDeftMasked = -1.0e6f;
+constexpr int kDeftMaskGroups = 5;       // mask groups 128 consecutive query rows can touch (g = 1, mask_len 32: 4 + 1)
+
+template <typename E, int D>
+__global__ void __launch_bounds__(kWideBlock, D > 128 ? 1 : 2) deft_stage1_kernel(DeftArgs d) {
+  using W = WideGeom<D>;
+  const Stage1Args& a = d.s;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int subtree = blockIdx.x / a.hkv;
+  const int kvh = blockIdx.x - subtree * a.hkv;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const VnodeView vn = load_vnode<false>(a, subtree);
+  const int rows_total = vn.q_len * a.g;
+  const int64_t* masks = d.causalmask + d.causalmask_offset[subtree];
+  const int grp_row = lane / W::kChunks, pos = lane % W::kChunks;
+  const char* kbase = a.k + 2 * ((int64_t)kvh * a.sk1);
+  const char* vbase = a.v + 2 * ((int64_t)kvh * a.sv1);
+  const unsigned k_stride = (unsigned)(2 * a.sk0), v_stride = (unsigned)(2 * a.sv0);
+  const unsigned ring = lds_offset(smem);
+  // the mask words of the chunk in LDS, after the ring: [kDeftMaskGroups][kDeftChunk] 64-bit words
+  uint32_t* mask_lds = reinterpret_cast<uint32_t*>(smem + W::kRing);
+  const unsigned mask_lds_addr = ring + W::kRing;
+  WideLane la0;
+  init_lane<D>(la0, ring);
+  const int nchunks = (vn.kv_len + kDeftChunk - 1) / kDeftChunk;
+  const int h = lane >> 5;
+
+  for (int row0 = 0; row0 < rows_total; row0 += kWideRows) {
+    const int my_row0 = row0 + 32 * wave;
+    const bool active = my_row0 < rows_total;
+    const char* q_src = q_row_address32<false>(a, vn, kvh, active ? my_row0 : rows_total);
+    u32x4 qf[D / 16];
+    load_q_frags32<D>(q_src, qf);
+    WideState<D> st;
+    reset_state<D>(st);
+    // the lane's request within the subtree's query set, its mask group and its bit in the group's words
+    const int my_req = min(my_row0 + (lane & 31), rows_total - 1) / a.g;
+    const int first_group = (row0 / a.g) / d.mask_len;
+    const int groups_here = min((min(row0 + kWideRows, rows_total) - 1) / a.g / d.mask_len - first_group + 1, kDeftMaskGroups);
+    const int my_group = min(my_req / d.mask_len - first_group, kDeftMaskGroups - 1);
+    const int my_bit = my_req & (d.mask_len - 1);
+    const bool upper = my_bit >= 32;
+    const unsigned bit = 1u << (my_bit & 31);
+    for (int chunk = 0; chunk < nchunks; ++chunk) {
+      const int c0 = chunk * kDeftChunk;
+      const int here = min(kDeftChunk, vn.kv_len - c0);
+      __syncthreads();   // the previous pass (or chunk) is out of LDS
+      if (row0 == 0 || nchunks > 1) {
+        // K and V rows of the chunk: 2 x 16 groups of 1 KB per super tile, dealt to the four waves
+        // (tokens past the end repeat the last one: their scores are masked)
+#pragma unroll
+        for (int sup = 0; sup < 2; ++sup)
+#pragma unroll
+          for (int u = 0; u < W::kUnits; ++u) {
+            const bool is_v = W::kGroups >= kWideWaves ? u >= W::kSlots : wave >= W::kGroups;
+            const int sl = u % W::kSlots;
+            const int grp = W::kGroups >= kWideWaves ? sl * kWideWaves + wave : wave % W::kGroups;
+            const int row = grp * W::kGroupRows + grp_row;
+            const int t = min(c0 + sup * W::kTokens + row, vn.kv_len - 1);
+            const unsigned slot = (unsigned)a.kv_entries[vn.kv_base + t];
+            const char* src = (is_v ? vbase : kbase) + (uint64_t)slot * (is_v ? v_stride : k_stride);
+            load_direct16(src + 16 * (pos ^ W::swz(row)), ring + sup * W::kBytes + (is_v ? W::kBytesK : 0) + grp * 1024);
+          }
+      }
+      // the mask words of this pass's groups for the chunk's tokens (zero past the subtree)
+      for (int i = threadIdx.x; i < groups_here * kDeftChunk; i += kWideBlock) {
+        const int gsel = i / kDeftChunk, t = i - gsel * kDeftChunk;
+        const int64_t word = t < here ? masks[(int64_t)(first_group + gsel) * vn.kv_len + c0 + t] : 0;
+        mask_lds[2 * i] = (uint32_t)(uint64_t)word;
+        mask_lds[2 * i + 1] = (uint32_t)((uint64_t)word >> 32);
+      }
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): rows landed (and the Q fragments)
+      __syncthreads();
+      if (active) {
+        const int tiles = (here + kTileTokens - 1) / kTileTokens;
+        for (int tile = 0; tile < tiles; ++tile) {
+          // the lane's 16 tokens of the tile are four runs of four consecutive ones: 32 bytes of mask words each
+          const unsigned words = mask_lds_addr + 8u * (unsigned)(my_group * kDeftChunk + tile * kTileTokens + 4 * h);
+          auto mask = [&](f32x16& sc) {
+#pragma unroll
+            for (int quad = 0; quad < 4; ++quad) {
+              const u32x4 w0 = lds_read16(words + 64u * quad), w1 = lds_read16(words + 64u * quad + 16u);
+              const unsigned m4[4] = {upper ? w0[1] : w0[0], upper ? w0[3] : w0[2], upper ? w1[1] : w1[0], upper ? w1[3] : w1[2]};
+#pragma unroll
+              for (int jj = 0; jj < 4; ++jj) sc[4 * quad + jj] = (m4[jj] & bit) ? sc[4 * quad + jj] : kDeftMasked;
+            }
+          };
+          const WideLane la = at_buffer(la0, (unsigned)(tile >> 1) * W::kBytes);
+          tile_step32<E, D>(la, (tile & 1) * W::kTileBytes, here - tile * kTileTokens, a.scale_log2, qf, st, mask);
+        }
+      }
+    }
+    finish_state<D>(st);
+    // (the reference rounds the normalised partial output to fp16 before it stores it, DeFT.py:391)
+    if (active) write_partials32<D, true>(a, vn, kvh, my_row0, st);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // Stage 2
 // ---------------------------------------------------------------------------------------
 struct Stage2Args {
@@ -1668,6 +1804,42 @@ int launch_stage2(const Stage2Args& a, int d, int dtype, hipStream_t stream) {
     case 128: return launch_stage2_inst<E, 128>(a, stream);    \
     case 256: return launch_stage2_inst<E, 256>(a, stream);    \
     default: return FT_ERR_HEAD_DIM;                           \
+  }
+  if (dtype == FT_DTYPE_F16) { FT_DISPATCH_D(F16) }
+  if (dtype == FT_DTYPE_BF16) { FT_DISPATCH_D(BF16) }
+#undef FT_DISPATCH_D
+  return FT_ERR_DTYPE;
+}
+
+template <typename E, int D>
+int launch_deft_inst(const DeftArgs& d, hipStream_t stream) {
+  constexpr size_t lds = (size_t)WideGeom<D>::kLds;
+  static_assert(kDeftMaskGroups * kDeftChunk * 8 <= 4 * WideGeom<D>::kIdxCap, "the mask words share the index area");
+  auto kern = deft_stage1_kernel<E, D>;
+  static std::atomic<bool> configured_on[kMaxDevices];
+  std::atomic<bool>& configured = configured_on[current_device()];
+  if (!configured.load(std::memory_order_acquire)) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+      (void)hipGetLastError();
+      return FT_ERR_LAUNCH;
+    }
+    configured.store(true, std::memory_order_release);
+  }
+  const int64_t blocks = (int64_t)d.num_subtrees * d.s.hkv;
+  if (blocks == 0) return FT_OK;
+  if (blocks > INT32_MAX) return FT_ERR_ARGUMENT;
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks, 1, 1), dim3(kWideBlock, 1, 1), lds, stream, d);
+  return hipGetLastError() == hipSuccess ? FT_OK : FT_ERR_LAUNCH;
+}
+
+int launch_deft(const DeftArgs& d, int head_dim, int dtype, hipStream_t stream) {
+#define FT_DISPATCH_D(E)                                         \
+  switch (head_dim) {                                            \
+    case 32: return launch_deft_inst<E, 32>(d, stream);          \
+    case 64: return launch_deft_inst<E, 64>(d, stream);          \
+    case 128: return launch_deft_inst<E, 128>(d, stream);        \
+    case 256: return launch_deft_inst<E, 256>(d, stream);        \
+    default: return FT_ERR_HEAD_DIM;                             \
   }
   if (dtype == FT_DTYPE_F16) { FT_DISPATCH_D(F16) }
   if (dtype == FT_DTYPE_BF16) { FT_DISPATCH_D(BF16) }
@@ -1977,6 +2149,60 @@ int ft_decode(const void* q, const void* k, const void* v, void* o,
                                 vnode_to_kv_lens, vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, mid_o, so0, so1,
                                 mid_lse, sl0, phase_node_nums, phase_node_offsets, phase_q_tile_sizes,
                                 phase_kv_tile_sizes, num_qo_heads, num_kv_heads, head_dim, sm_scale, dtype, stream))
+    return rc;
+  return ft_stage2(req_to_vnode_entries, req_to_vnode_offs, req_to_vnode_lens, mid_o, so0, so1, mid_lse, sl0, o, oo0,
+                   oo1, batch_size, num_qo_heads, head_dim, dtype, stream);
+}
+
+int ft_deft_stage1(const void* q, const void* k, const void* v,
+                   int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+                   const int32_t* vnode_to_kv_entries, const int32_t* vnode_to_kv_offs,
+                   const int32_t* vnode_to_kv_lens, const int32_t* vnode_to_q_entries,
+                   const int32_t* vnode_to_q_offs, const int32_t* vnode_to_q_lens,
+                   const int64_t* causalmask, const int32_t* causalmask_offset,
+                   int subtree_num, int num_qo_heads, int num_kv_heads, int head_dim, int mask_len, float sm_scale,
+                   float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
+                   int dtype, ft_stream_t stream) {
+  if (num_kv_heads < 1 || num_qo_heads % num_kv_heads != 0) return FT_ERR_GROUP;
+  const int g = num_qo_heads / num_kv_heads;
+  if (int rc = check_common(head_dim, g, dtype)) return rc;
+  if (head_dim < 32) return FT_ERR_HEAD_DIM;
+  if (subtree_num == 0) return FT_OK;
+  DeftArgs d{};
+  if (int rc = stage1_setup(d.s, q, k, v, sq0, sq1, sk0, sk1, sv0, sv1, vnode_to_kv_entries, vnode_to_kv_offs,
+                            vnode_to_kv_lens, vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, num_kv_heads, g,
+                            head_dim, sm_scale, mid_o, so0, so1, mid_lse, sl0, dtype))
+    return rc;
+  if (!causalmask || !causalmask_offset) return FT_ERR_NULL_POINTER;
+  if (subtree_num < 0 || !range_ok(0, subtree_num, num_kv_heads)) return FT_ERR_ARGUMENT;
+  // a power of two of at most 64 requests per mask word, and few enough words per token for the
+  // 128 query rows a block serves at a time
+  if (mask_len < 1 || mask_len > 64 || (mask_len & (mask_len - 1)) != 0) return FT_ERR_ARGUMENT;
+  const int requests_per_pass = (kWideRows + g - 1) / g + 1;
+  if ((requests_per_pass + mask_len - 1) / mask_len + 1 > kDeftMaskGroups) return FT_ERR_ARGUMENT;
+  d.causalmask = causalmask;
+  d.causalmask_offset = causalmask_offset;
+  d.mask_len = mask_len;
+  d.num_subtrees = subtree_num;
+  return launch_deft(d, head_dim, dtype, stream);
+}
+
+int ft_deft_decode(const void* q, const void* k, const void* v, void* o,
+                   int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+                   int64_t oo0, int64_t oo1,
+                   const int32_t* vnode_to_kv_entries, const int32_t* vnode_to_kv_offs,
+                   const int32_t* vnode_to_kv_lens, const int32_t* vnode_to_q_entries,
+                   const int32_t* vnode_to_q_offs, const int32_t* vnode_to_q_lens,
+                   const int64_t* causalmask, const int32_t* causalmask_offset,
+                   const int32_t* req_to_vnode_entries, const int32_t* req_to_vnode_offs,
+                   const int32_t* req_to_vnode_lens,
+                   float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
+                   int subtree_num, int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
+                   int mask_len, float sm_scale, int dtype, ft_stream_t stream) {
+  if (int rc = ft_deft_stage1(q, k, v, sq0, sq1, sk0, sk1, sv0, sv1, vnode_to_kv_entries, vnode_to_kv_offs,
+                              vnode_to_kv_lens, vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, causalmask,
+                              causalmask_offset, subtree_num, num_qo_heads, num_kv_heads, head_dim, mask_len, sm_scale,
+                              mid_o, so0, so1, mid_lse, sl0, dtype, stream))
     return rc;
   return ft_stage2(req_to_vnode_entries, req_to_vnode_offs, req_to_vnode_lens, mid_o, so0, so1, mid_lse, sl0, o, oo0,
                    oo1, batch_size, num_qo_heads, head_dim, dtype, stream);

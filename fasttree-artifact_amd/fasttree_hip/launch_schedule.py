@@ -80,6 +80,11 @@ TILE_US_ALONE = 0.95
 #: Bytes per microsecond the narrow vnodes stream at most on DEFAULT_COMPUTE_UNITS units (rows of
 #: 2 * head_dim bytes at random slots); taken to scale with the number of units.
 NARROW_BYTES_PER_US = 5.6e6
+#: What a launch costs before its first block runs and after its last one ends, as seen between two
+#: events on the launch stream (measured on launches of a few vnodes: 15 us between events where the
+#: blocks themselves model at 12).  Part of the reported duration only: it is the same for every
+#: layout of a launch, so the choice between layouts does not see it.
+LAUNCH_US = 3.0
 #: A tile step of a piece of at most 64 query rows, relative to one of a full block.  The block's
 #: waves then split the tokens of a super tile, but the super tile is loaded all the same: fitted on
 #: the programs of an irregular tree of 500 requests, 1.21 against 1.44 us per tile step.
@@ -130,6 +135,10 @@ class LaunchPhases(list):
     prog_table = None
     num_programs = 0
     narrow_in_programs = 0
+    #: what the schedule's model expects the first-stage launch to take, and the machine it was laid out for
+    modelled_us = None
+    num_cus = None
+    block_slots = None
 
 
 @dataclass
@@ -617,7 +626,7 @@ def _block_programs(runs, batch_size, group, num_kv_heads, *,
                 phase_node_nums=[n_wide, len(new_kv_offs) - n_wide], phase_node_offsets=[0, n_wide],
                 prog_table=i32(prog_table).reshape(-1, 4), narrow_in_programs=narrow_first,
                 program_tiles=np.asarray(program_tiles, dtype=np.float64), block_slots=int(block_slots),
-                modelled_us=float(modelled), num_cus=int(num_cus),
+                modelled_us=float(modelled) + LAUNCH_US, num_cus=int(num_cus),
             )
 
         return float(modelled), build

@@ -536,6 +536,7 @@ def fasttree_preparation(
         per_request = (sched.req_entries, sched.req_offs, sched.req_lens)
         rows = sched.num_rows
         phase_nums, phase_offs = LaunchPhases(sched.phase_node_nums), list(sched.phase_node_offsets)
+        phase_nums.modelled_us, phase_nums.num_cus, phase_nums.block_slots = sched.modelled_us, sched.num_cus, sched.block_slots
         if sched.num_programs > 0:
             phase_nums.prog_table = place("prog_table", sched.prog_table.reshape(-1))
             phase_nums.num_programs = sched.num_programs

@@ -8,10 +8,13 @@ Engines (``--choice``): ``fasttree`` is the tree decode (planner + the two HIP s
 ``[B, max_seqlen, Hkv, D]`` (the layout of kernel_bench/flash_attn_wrap.py:36-70), here a HIP
 kernel of this library, and it is the result the tree decode is checked against with the
 reference's criterion ``allclose(rtol=1e-2, atol=1e-2)`` (kernel_bench/benchmark.py:216-220).
-``DeFT`` is DeFT-Flatten's schedule -- the depth-first token order cut into subtrees of 128 tokens,
-one thread block per (subtree, kv head), kernel_bench/DeFT.py:14-135 and benchmark.py:180-211 --
-run through this library's kernels as block programs (``deft_schedule.py``); it is checked against
-the gathered decode like the tree decode.  The reference's other engines (SGLang Triton,
+``DeFT`` is DeFT-Flatten as the reference benchmarks it (kernel_bench/DeFT.py, benchmark.py:180-211):
+the depth-first token order cut into subtrees of 128 tokens, one thread block per (subtree, kv
+head) over the subtree's whole query set with a 64-bit mask word per token and group of 64
+requests, reading the per-request gathered cache -- this library's ``DeFT.py`` on its own HIP
+kernel; it is checked against the gathered decode like the tree decode.  ``DeFT_schedule`` runs the
+same partition through the *tree* kernels instead (one vnode per node piece, ``deft_schedule.py``;
+kept for comparison, not part of ``all``).  The reference's other engines (SGLang Triton,
 FlashInfer) are Triton / CUDA libraries and have no counterpart here.
 
 Timing follows the method of ``triton.testing.do_bench`` as the reference calls it
@@ -34,11 +37,12 @@ import torch
 sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), ".."))
 
 from fasttree_hip import planner as _planner  # noqa: E402
-from fasttree_hip.decode import fasttree_decode, gathered_decode  # noqa: E402
+from fasttree_hip.decode import fasttree_decode, fasttree_decode_stage1, gathered_decode  # noqa: E402
 from fasttree_hip.inputs import qkv_preparation  # noqa: E402
 from fasttree_hip.kv_tree import retrive_from_file  # noqa: E402
 from fasttree_hip.planner import FastTreeParams, fasttree_preparation  # noqa: E402
 from deft_schedule import deft_preparation  # noqa: E402
+from DeFT import DeFT_decode, DeFT_preparation  # noqa: E402
 
 QUANTILES = [0.5, 0.2, 0.8]
 
@@ -161,18 +165,51 @@ def main(args):
             return out_tree
 
         out_tree_attn = run_and_bench(call_tree_attn, "fasttree attn").cpu()
+        modelled = getattr(fasttree_aux[11], "modelled_us", None)
+        if modelled is not None and not args.signature:
+            # what the launch schedule's model expects of the first-stage launch beside what it takes: the
+            # median over back-to-back launches (warm caches, as the model's constants were measured)
+            def call_stage1():
+                fasttree_decode_stage1(Q, K_tree_tensor, V_tree_tensor, *fasttree_aux[:6], sm_scale, fasttree_aux[9],
+                                       fasttree_aux[10], fasttree_aux[11], fasttree_aux[12], q_tiles, kv_tiles)
+
+            for _ in range(20):
+                call_stage1()
+            marks = [torch.cuda.Event(enable_timing=True) for _ in range(61)]
+            marks[0].record()
+            for i in range(60):
+                call_stage1()
+                marks[i + 1].record()
+            torch.cuda.synchronize()
+            measured = torch.tensor([a.elapsed_time(b) for a, b in zip(marks, marks[1:])]).median().item() * 1e3
+            print(f"fasttree stage 1: modelled {modelled:.1f} us, measured {measured:.1f} us between events (warm), "
+                  f"{fasttree_aux[11].num_programs} programs on {fasttree_aux[11].block_slots} block slots", flush=True)
+            results["stage1_modelled_us"], results["stage1_measured_us"] = float(modelled), float(measured)
 
     out_deft_attn = None
     if args.choice in ["DeFT", "all"]:
-        subtree_len = 128  # (kernel_bench/benchmark.py:183)
-        deft_aux = deft_preparation(tree_info, KV_ptrs, batch_size, num_qo_heads, num_kv_heads, head_dim, subtree_len)
+        subtree_len, mask_len = 128, 64  # (kernel_bench/benchmark.py:183-184)
+        deft_aux = DeFT_preparation(tree_info, K_cache, subtree_len, mask_len, num_qo_heads, head_dim)
         out_deft = torch.empty(batch_size, num_qo_heads, head_dim, device="cuda", dtype=dtype)
+        k_flat = K_cache.view(-1, K_cache.shape[-2], K_cache.shape[-1])
+        v_flat = V_cache.view(-1, V_cache.shape[-2], V_cache.shape[-1])
 
         def call_deft_attn():
-            fasttree_decode(Q, K_tree_tensor, V_tree_tensor, out_deft, *deft_aux, [1, 1], [32, 32], sm_scale)
+            DeFT_decode(Q, k_flat, v_flat, out_deft, *deft_aux, Q_TILE_SIZE_PER_PHASE[0], KV_TILE_SIZE_PER_PHASE[0],
+                        sm_scale, mask_len)
             return out_deft
 
         out_deft_attn = run_and_bench(call_deft_attn, "DeFT attn").cpu()
+
+    if args.choice == "DeFT_schedule":
+        sched_aux = deft_preparation(tree_info, KV_ptrs, batch_size, num_qo_heads, num_kv_heads, head_dim, 128)
+        out_sched = torch.empty(batch_size, num_qo_heads, head_dim, device="cuda", dtype=dtype)
+
+        def call_deft_schedule():
+            fasttree_decode(Q, K_tree_tensor, V_tree_tensor, out_sched, *sched_aux, [1, 1], [32, 32], sm_scale)
+            return out_sched
+
+        run_and_bench(call_deft_schedule, "DeFT schedule")
 
     if out_flash_attn is not None and out_deft_attn is not None:
         ok = torch.allclose(out_flash_attn, out_deft_attn, rtol=1e-2, atol=1e-2)
@@ -207,7 +244,7 @@ def build_parser():
     parser.add_argument("--num_kv_heads", type=int, default=32)
     parser.add_argument("--head_dim", type=int, default=128)
     parser.add_argument("--signature", type=str, default=None)
-    parser.add_argument("--choice", type=str, choices=["flash_attn", "fasttree", "DeFT", "all"], default="all")
+    parser.add_argument("--choice", type=str, choices=["flash_attn", "fasttree", "DeFT", "DeFT_schedule", "all"], default="all")
     parser.add_argument("--profile", action="store_true", default=False)
     parser.add_argument("--mi355x", action="store_true", default=False,
                         help="query tiles, parallelism thresholds and KV split sizes for MI355X instead of the H100 defaults, "

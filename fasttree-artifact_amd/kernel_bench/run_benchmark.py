@@ -5,8 +5,8 @@ of the tree decode (gamma = 10 with one KV split: every request its own full pat
 gamma = -10: never merge, "w/o greedy"), and the never-merge plan without KV splits
 ("node-wise": every tree node one batched attention over its own KV, merged per request -- the
 schedule of a multi-level cascade attention, which the reference measures with FlashInfer,
-kernel_bench/bench_cascade.py), and DeFT-Flatten's schedule (subtrees of 128 tokens of the
-depth-first token order, kernel_bench/DeFT.py) as block programs through the same kernels.
+kernel_bench/bench_cascade.py), and DeFT-Flatten (subtrees of 128 tokens of the depth-first token
+order, one block per subtree with a mask word per token, kernel_bench/DeFT.py) on its own kernel.
 
     python run_benchmark.py --out sweep --preset mi355x [--cases 0,8,9] [--heads "32 8"]
 
@@ -92,6 +92,8 @@ def run_case(out_dir, nodes, contexts, q_heads, k_heads, preset, log=print, extr
                 row["check"] = res.get("check")
                 row["max_abs"] = res.get("max_abs")
                 row["mean_abs"] = res.get("worst_request_mean_abs")
+                row["modelled_us"] = res.get("stage1_modelled_us")
+                row["measured_us"] = res.get("stage1_measured_us")
             else:
                 row[tag] = next(iter(v for k, v in res.items() if k.startswith("fasttree")), None)
     log(f"{row['tree']:60s} {row['heads']:6s} {preset:9s} gathered {row['flash_attn']:.4f} ms  tree {row['fasttree']:.4f} ms  "
@@ -103,7 +105,7 @@ def run_case(out_dir, nodes, contexts, q_heads, k_heads, preset, log=print, extr
 def write_table(rows, path):
     engines = ["flash_attn", "naive", "deft", "node_wise", "no_greedy", "fasttree"]
     with open(path, "w") as fh:
-        fh.write("| tree (nodes / tokens per level) | q/kv heads | preset | gathered ms | tree, naive ms | DeFT schedule ms | node-wise ms | tree, w/o greedy ms | tree ms | "
+        fh.write("| tree (nodes / tokens per level) | q/kv heads | preset | gathered ms | tree, naive ms | DeFT ms | node-wise ms | tree, w/o greedy ms | tree ms | "
                  "speed-up over gathered | normalised: gathered / naive / DeFT / node-wise / w/o greedy / tree | allclose 1e-2 | max abs | worst request mean abs |\n")
         fh.write("|---|---|---|---|---|---|---|---|---|---|---|---|---|---|\n")
         for r in rows:
@@ -119,7 +121,24 @@ def write_table(rows, path):
             best = sum(1 for r in part if r["fasttree"] <= 1.05 * min(r[e] for e in engines))
             fh.write(f"Preset `{preset}`: {len(part)} cases, geometric-mean speed-up of the tree decode over the gathered "
                      f"decode {geo:.2f}x; the tree decode is the fastest engine (within 5 %) in {best} of them; "
-                     f"{sum(1 for r in part if not (r['check'] and r['deft_check']))} failed the allclose check (tree decode or DeFT schedule).\n\n")
+                     f"{sum(1 for r in part if not (r['check'] and r['deft_check']))} failed the allclose check (tree decode or DeFT).\n\n")
+
+
+def write_model_check(rows, path):
+    """The launch schedule's modelled duration of the first-stage launch beside the measured one
+    (warm, between events on the launch stream: the kernel plus 2-4 us of launch gap), for the
+    cases whose lists were arranged as block programs."""
+    rows = [r for r in rows if r.get("modelled_us") is not None]
+    with open(path, "w") as fh:
+        fh.write("| tree (nodes / tokens per level) | q/kv heads | modelled us | measured us | modelled / measured |\n|---|---|---|---|---|\n")
+        for r in rows:
+            fh.write(f"| {r['tree']} | {r['heads']} | {r['modelled_us']:.1f} | {r['measured_us']:.1f} | {r['modelled_us'] / r['measured_us']:.2f} |\n")
+        if rows:
+            ratios = [r["modelled_us"] / r["measured_us"] for r in rows]
+            geo = math.exp(sum(math.log(x) for x in ratios) / len(ratios))
+            inside = sum(1 for x in ratios if 0.8 <= x <= 1.2)
+            fh.write(f"\n{len(rows)} launches: modelled / measured between {min(ratios):.2f} and {max(ratios):.2f}, geometric mean "
+                     f"{geo:.2f}; {inside} within 20 % of the measured time.\n")
 
 
 def main(argv=None):
@@ -145,6 +164,7 @@ def main(argv=None):
                                      log=lambda *a: print(*a, flush=True), extra=args.extra.split(),
                                      outputs=outputs[preset]))
                 write_table(rows, os.path.join(args.out, "results.md"))
+                write_model_check(rows, os.path.join(args.out, "model_check.md"))
     failed = [r for r in rows if not (r["check"] and r["deft_check"])]
     print(f"{len(rows)} cases, {len(failed)} failed the allclose check", flush=True)
     return 1 if failed else 0

@@ -214,6 +214,44 @@ int ft_gathered_decode(const void* q, const void* k_cache, const void* v_cache,
                        float* mid_o, float* mid_lse, int dtype, ft_stream_t stream);
 
 /*
+ * DeFT-Flatten, the tree-attention engine the reference's benchmark compares itself with
+ * (kernel_bench/DeFT.py): ft_deft_stage1 replaces _fwd_DeFT_decode_stage1 / _DeFT_attn_stage_1
+ * (DeFT.py:194-403), ft_deft_decode the whole of DeFT_decode (DeFT.py:489-560; its second stage,
+ * DeFT.py:406-486, is the arithmetic of ft_stage2).  A vnode here is a subtree: a run of
+ * consecutive tokens of the depth-first token order that may span several tree nodes
+ * (vnode_to_kv_*), with the sorted set of requests that attend any of them (vnode_to_q_*).
+ * causalmask holds, per subtree from causalmask_offset[subtree] on, kv_len 64-bit words for every
+ * group of mask_len consecutive requests of the subtree's set: bit r of word t of group m says
+ * that request m * mask_len + r of the set attends token t (DeFT.py:96-113).  One block per
+ * (subtree, KV head); scores of tokens a request does not attend are set to a large negative value
+ * before the soft-max; the normalised partial output is rounded to fp16 before it is stored to the
+ * fp32 mid_o, as in the reference (DeFT.py:391).  mask_len is a power of two, at most 64, and at
+ * least 128 / (3 * g) (the benchmark uses 64); head_dim in {32, 64, 128, 256}.
+ */
+int ft_deft_stage1(const void* q, const void* k, const void* v,
+                   int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+                   const int32_t* vnode_to_kv_entries, const int32_t* vnode_to_kv_offs,
+                   const int32_t* vnode_to_kv_lens, const int32_t* vnode_to_q_entries,
+                   const int32_t* vnode_to_q_offs, const int32_t* vnode_to_q_lens,
+                   const int64_t* causalmask, const int32_t* causalmask_offset,
+                   int subtree_num, int num_qo_heads, int num_kv_heads, int head_dim, int mask_len, float sm_scale,
+                   float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
+                   int dtype, ft_stream_t stream);
+
+int ft_deft_decode(const void* q, const void* k, const void* v, void* o,
+                   int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
+                   int64_t oo0, int64_t oo1,
+                   const int32_t* vnode_to_kv_entries, const int32_t* vnode_to_kv_offs,
+                   const int32_t* vnode_to_kv_lens, const int32_t* vnode_to_q_entries,
+                   const int32_t* vnode_to_q_offs, const int32_t* vnode_to_q_lens,
+                   const int64_t* causalmask, const int32_t* causalmask_offset,
+                   const int32_t* req_to_vnode_entries, const int32_t* req_to_vnode_offs,
+                   const int32_t* req_to_vnode_lens,
+                   float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
+                   int subtree_num, int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
+                   int mask_len, float sm_scale, int dtype, ft_stream_t stream);
+
+/*
  * The decode step's new K and V rows [num_tokens, Hkv, D] written to the pools at the slots
  * out_cache_loc[t] (int32, or int64 when loc_is_int64), both tensors in one launch on `stream`:
  * the two indexed assignments of SGLang v0.2.13's RadixAttention.store_kv_cache, which the hook

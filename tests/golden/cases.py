@@ -191,3 +191,50 @@ def kernel_case_inputs(case, tree, ptrs, batch):
     v = draw((total, case["Hkv"], case["D"]))
     q = draw((batch, case["Hq"], case["D"]))
     return q, k, v
+
+
+def _deft_cases():
+    """Trees for the comparison engine (DeFT-Flatten): subtrees that span several nodes and nodes
+    that span several subtrees, query sets of more than one mask word (more than 64 requests) and
+    of more than one pass of a thread block (more than 128 query rows), MHA and GQA.  ``q_tile``
+    is the reference kernel's Q_TILE_SIZE (a divisor of mask_len)."""
+    def case(name, tree, hq, hkv, d, seed, subtree_len=128, mask_len=64, q_tile=16):
+        return dict(name=name, tree=tree, Hq=hq, Hkv=hkv, D=d, dtype="fp16", seed=seed, subtree_len=subtree_len,
+                    mask_len=mask_len, q_tile=q_tile)
+    return [
+        case("kat1_mha", regular([1, 1, 2], [100, 50, 10]), 4, 4, 64, 31, subtree_len=32),
+        case("two_level_gqa4", regular([1, 6], [200, 37]), 8, 2, 128, 32),
+        case("three_level_gqa4", regular([1, 3, 24], [150, 70, 19]), 8, 2, 128, 33),
+        case("irregular_gqa8", irregular(5, levels=4, fanout_range=(1, 4), len_range=(4, 90), max_leaves=40), 16, 2, 128, 35),
+        case("many_requests_gqa4", regular([1, 2, 70], [50, 30, 7]), 8, 2, 64, 36, subtree_len=64),
+        case("mha_d32_two_words", regular([1, 90], [40, 5]), 2, 2, 32, 37),
+    ]
+
+
+DEFT_CASES = _deft_cases()
+
+
+def gathered_cache(tree, ptrs, k_pool, v_pool):
+    """The per-request gathered, zero-padded caches ``[B, max_seqlen, Hkv, D]`` of
+    kernel_bench/flash_attn_wrap.py:36-67 from a node-major pool (CPU tensors)."""
+    import torch
+
+    paths = {}
+    for index, node in enumerate(tree):
+        if node.num_children == 0:
+            chain, cur = [], index
+            while cur >= 0:
+                chain.append(cur)
+                cur = tree[cur].parent
+            for r in node.requests:
+                paths[r] = list(reversed(chain))
+    batch = len(paths)
+    tokens = [np.concatenate([np.arange(ptrs[n], ptrs[n + 1]) for n in paths[r]]) for r in range(batch)]
+    width = max(len(t) for t in tokens)
+    k_cache = torch.zeros((batch, width) + tuple(k_pool.shape[1:]), dtype=k_pool.dtype)
+    v_cache = torch.zeros_like(k_cache)
+    for r, t in enumerate(tokens):
+        idx = torch.from_numpy(t.astype(np.int64))
+        k_cache[r, : len(t)] = k_pool[idx]
+        v_cache[r, : len(t)] = v_pool[idx]
+    return k_cache, v_cache

@@ -6,7 +6,7 @@ Run once in a container that holds the reference checkout; the fixtures it write
 plain data (JSON / npz) and are what the tests read -- nothing in the test suite, the
 smoke run or the bench imports the reference.
 
-    python tests/golden/make_goldens.py [--reference /root/reference] [--only planner|kernel]
+    python tests/golden/make_goldens.py [--reference /root/reference] [--only planner|kernel|deft]
 
 What is taken from the reference: ``_tree_heuristic``, ``fasttree_preparation``,
 ``FastTreeParams`` and ``fasttree_decode`` of kernel_bench/fasttree.py.  Because that
@@ -14,6 +14,11 @@ planner hard-wires ``torch.device("cuda")`` for its output tensors
 (kernel_bench/fasttree.py:265), the module's ``torch`` name is pointed at a thin proxy
 whose ``device()`` is a no-op context so the tensors land on the CPU; nothing else is
 altered.  Inputs (trees, requests, Q/K/V) are built by this repository's own generators.
+
+``--only deft`` writes ``deft_*.npz``: the index arrays and masks of the reference's
+``DeFT_preparation`` and the outputs of its ``DeFT_decode`` (kernel_bench/DeFT.py, the comparison
+engine of the reference's benchmark) under the same interpreter, on the per-request gathered
+cache that engine reads.
 """
 
 from __future__ import annotations
@@ -163,12 +168,73 @@ def kernel_goldens(ref, out_dir: str, names=None):
         print(f"kernel {case['name']}: {time.time() - t0:.1f}s", file=sys.stderr)
 
 
+def load_reference_deft(ref_root: str):
+    os.environ["TRITON_INTERPRET"] = "1"
+    import torch
+
+    bench_dir = os.path.join(ref_root, "kernel_bench")
+    sys.path.insert(0, bench_dir)            # DeFT.py imports kv_tree_simple from its own directory
+    try:
+        spec = importlib.util.spec_from_file_location("_reference_deft", os.path.join(bench_dir, "DeFT.py"))
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+    finally:
+        sys.path.remove(bench_dir)
+
+    class _HostTorch:
+        def __getattr__(self, name):
+            return getattr(torch, name)
+
+        @staticmethod
+        def device(*_a, **_k):
+            return contextlib.nullcontext()
+
+    mod.torch = _HostTorch()
+    return mod
+
+
+def deft_goldens(ref_root: str, out_dir: str):
+    import torch
+
+    from cases import DEFT_CASES, gathered_cache
+
+    ref = load_reference_deft(ref_root)
+    names = ["vnode_to_kv_entries", "vnode_to_kv_offs", "vnode_to_kv_lens", "vnode_to_q_entries", "vnode_to_q_offs",
+             "vnode_to_q_lens", "causalmask", "causalmask_offset", "req_to_vnode_entries", "req_to_vnode_offs",
+             "req_to_vnode_lens"]
+    for case in DEFT_CASES:
+        t0 = time.time()
+        tree, ptrs, batch = build_tree(case["tree"])
+        q, k_pool, v_pool = kernel_case_inputs(case, tree, ptrs, batch)
+        k_cache, v_cache = gathered_cache(tree, ptrs, k_pool, v_pool)
+        ref.cur_length = 0                   # (a module global the partition accumulates in, DeFT.py:26)
+        aux = ref.DeFT_preparation(tree, k_cache, case["subtree_len"], case["mask_len"], case["Hq"], case["D"])
+        o = torch.zeros_like(q)
+        sm_scale = 1.0 / (case["D"] ** 0.5)
+        ref.DeFT_decode(q, k_cache.view(-1, case["Hkv"], case["D"]), v_cache.view(-1, case["Hkv"], case["D"]), o, *aux,
+                        case["q_tile"], 32, sm_scale, case["mask_len"])
+        record = {name: t.numpy() for name, t in zip(names, aux[:11])}
+        np.savez_compressed(
+            os.path.join(out_dir, f"deft_{case['name']}.npz"),
+            o=o.view(torch.int16).numpy(), mid_o=aux[11].numpy(), mid_lse=aux[12].numpy(),
+            q_sha256=np.array(digest(q.view(torch.int16).numpy())),
+            k_sha256=np.array(digest(k_cache.view(torch.int16).numpy())),
+            v_sha256=np.array(digest(v_cache.view(torch.int16).numpy())),
+            **record,
+        )
+        print(f"deft {case['name']}: {time.time() - t0:.1f}s, {len(aux[1])} subtrees", file=sys.stderr)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--reference", default="/root/reference")
-    ap.add_argument("--only", choices=["planner", "kernel"], default=None)
+    ap.add_argument("--only", choices=["planner", "kernel", "deft"], default=None)
     ap.add_argument("--cases", default=None, help="kernel cases to (re)write, comma separated (default: all)")
     args = ap.parse_args()
+    if args.only in (None, "deft"):
+        deft_goldens(args.reference, HERE)
+        if args.only == "deft":
+            return
     ref = load_reference(args.reference)
     if args.only in (None, "planner"):
         with open(os.path.join(HERE, "planner_goldens.json"), "w") as fh:

@@ -21,7 +21,7 @@ def declared_symbols():
 
 def test_header_symbols_are_exported():
     names = declared_symbols()
-    assert names == ["ft_decode", "ft_decode_programs", "ft_decode_static", "ft_error_string", "ft_gathered_decode", "ft_stage1",
+    assert names == ["ft_decode", "ft_decode_programs", "ft_decode_static", "ft_deft_decode", "ft_deft_stage1", "ft_error_string", "ft_gathered_decode", "ft_stage1",
                      "ft_stage1_phases", "ft_stage1_programs", "ft_stage2", "ft_static_scratch_bytes", "ft_store_kv", "ft_version"]
     lib = ctypes.CDLL(_lib.LIB_PATH)
     for name in names:

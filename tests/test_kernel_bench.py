@@ -88,7 +88,7 @@ def test_plot_script_reads_the_sweep_table_and_draws_it(tmp_path):
     got = plot_norm_perf.read_table(str(table), "mi355x")
     assert len(got) == 4 and all(r["preset"] == "mi355x" for r in got)
     assert all(column in got[0] for column, _, _ in plot_norm_perf.ENGINES)
-    assert float(got[0]["tree ms"]) == 0.05 and float(got[0]["DeFT schedule ms"]) == 0.125
+    assert float(got[0]["tree ms"]) == 0.05 and float(got[0]["DeFT ms"]) == 0.125
     out = tmp_path / "r.png"
     assert plot_norm_perf.main(["--input", str(table), "--preset", "mi355x", "--output", str(out)]) == 0
     assert out.stat().st_size > 10000
