@@ -122,6 +122,13 @@ DEALT_MARGIN = 1.06
 LIGHT_WORK = 4096
 LIGHT_ROWS = 64
 NARROW_ROWS = 16
+#: Long narrow runs are cut (at multiples of a tile) while the launch's narrow vnodes would leave
+#: more than a quarter of the wave slots idle: a wave walks its run tile by tile, one memory round
+#: trip each, so a launch of a few long runs (a 1024-token prompt under 16 requests of a
+#: 32-head model: 32 waves that matter) lasts as long as its longest walk.  Pieces are not made
+#: shorter than this many tokens (every piece costs a start-up and a scratch row per request).
+NARROW_MIN_PIECE_TOKENS = 128
+NARROW_FILL = 0.75
 
 
 class LaunchPhases(list):
@@ -298,6 +305,34 @@ def block_programs(kv_offs, kv_lens, q_offs, q_lens, q_entries, batch_size, grou
     return _block_programs(runs, batch_size, group, num_kv_heads, num_cus=cus,
                            block_rows=block_rows, block_slots=block_slots, recut=recut, embed=embed, head_dim=head_dim,
                            layout=layout, cuts=cuts)[1]()
+
+
+def _cut_long_narrow_runs(narrow, group, heads, wave_slots):
+    """Narrow vnodes ``(kv_off, kv_len, requests)`` with the longest runs halved, again and again,
+    while the waves they take (one per 16 query rows and kv head) fill less than
+    :data:`NARROW_FILL` of the wave slots and the halves keep :data:`NARROW_MIN_PIECE_TOKENS`."""
+    import heapq
+
+    def waves(v):
+        return -(-len(v[2]) * group // NARROW_ROWS) * heads
+
+    total = sum(waves(v) for v in narrow)
+    heap = [(-v[1], i, v) for i, v in enumerate(narrow)]
+    heapq.heapify(heap)
+    serial = len(narrow)
+    whole = []                                          # runs that cannot be halved any more
+    while heap and total < NARROW_FILL * wave_slots and -heap[0][0] >= 2 * NARROW_MIN_PIECE_TOKENS:
+        length, index, v = heapq.heappop(heap)
+        length = -length
+        first = (length // 2 + TILE_TOKENS - 1) // TILE_TOKENS * TILE_TOKENS
+        if length - first < NARROW_MIN_PIECE_TOKENS:
+            whole.append((-length, index, v))
+            continue
+        for off, take in ((v[0], first), (v[0] + first, length - first)):
+            heapq.heappush(heap, (-take, serial, (off, take, v[2])))
+            serial += 1
+        total += waves(v)
+    return [v for _, _, v in sorted(heap + whole, key=lambda item: item[1])]
 
 
 def _resident_pieces(items, per_round, tiles, first_row):
@@ -521,7 +556,7 @@ def _block_programs(runs, batch_size, group, num_kv_heads, *,
         order = sorted(range(len(pieces)), key=lambda i: -pieces[i][3])
         programs = [[i] for i in order]
 
-    narrow_all = narrow
+    narrow_all = _cut_long_narrow_runs(narrow, group, heads, wave_slots)
 
     def finish(pieces, programs, overlap=False):
         # ---- narrow vnodes, longest first; dealt to the programs when those fill the machine

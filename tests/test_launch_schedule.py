@@ -155,11 +155,23 @@ def test_headline_tree_gets_a_block_per_piece_when_all_fit():
 
 def test_small_launches_keep_the_planner_chunks():
     """A launch whose programs would hold less than MIN_PROGRAM_TILES keeps the planner's KV
-    chunks, one vnode per program, longest first; a launch without wide vnodes has no programs."""
+    chunks, one vnode per program, longest first; a launch without wide vnodes has no programs,
+    and while its narrow vnodes would leave most wave slots idle its long runs are halved down to
+    pieces of 128 tokens (C1: 17 vnodes x 32 heads; the 1024-token root becomes 8 pieces)."""
     case = next(c for c in PLANNER_CASES if c["name"] == "c1")
     plan, batch, group, s = _schedule(case)
-    assert s.num_programs == 0 and s.phase_node_nums == [0, len(plan.vnode_to_kv_offs)]
-    assert sorted(zip(s.kv_offs.tolist(), s.kv_lens.tolist())) == sorted(zip(plan.vnode_to_kv_offs, plan.vnode_to_kv_lens))
+    assert s.num_programs == 0 and s.phase_node_nums == [0, 16 + 8]
+    want = sorted((o, n) for o, n in zip(plan.vnode_to_kv_offs, plan.vnode_to_kv_lens) if n != 1024) + []
+    root = [(o, n) for o, n in zip(plan.vnode_to_kv_offs, plan.vnode_to_kv_lens) if n == 1024]
+    assert len(root) == 1
+    want += [(root[0][0] + 128 * i, 128) for i in range(8)]
+    assert sorted(zip(s.kv_offs.tolist(), s.kv_lens.tolist())) == sorted(want)
+    assert s.num_rows == 16 + 8 * 16 and s.req_lens.tolist() == [9] * 16
+    # a launch that fills the wave slots keeps its runs whole
+    full = ls._cut_long_narrow_runs([(1000 * i, 600, [i]) for i in range(300)], 1, 8, 2048)
+    assert len(full) == 300
+    some = ls._cut_long_narrow_runs([(0, 600, [0, 1]), (600, 100, [2])], 4, 8, 2048)
+    assert sorted((o, n) for o, n, _ in some) == [(0, 160), (160, 160), (320, 280), (600, 100)]
     tree, ptrs, batch = build_tree({"kind": "regular", "sizes": [1, 64], "lens": [512, 32]})
     from fasttree_hip.planner import FastTreeParams, fasttree_plan
     p = FastTreeParams(); p.set_values(0.66, 0.33, 0.1); p.set_q_tile_sizes([16, 4]); p.set_kv_tile_sizes([32, 32]); p.set_kv_group_num(4)
