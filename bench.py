@@ -210,6 +210,7 @@ def main():
             sys.exit(2)
         from fasttree_hip.launch_schedule import LaunchPhases
         part = LaunchPhases([nums[0], 0] if args.phase == "wide" else [0, nums[1]])
+        part.narrow_table = getattr(nums, "narrow_table", None)
         if args.phase == "wide":
             part.prog_table = getattr(nums, "prog_table", None)
             part.num_programs = getattr(nums, "num_programs", 0)

@@ -140,6 +140,10 @@ struct Stage1Args {
   const int32_t* prog_table;
   int num_programs;
   int narrow_in_programs;          // narrow vnodes (from narrow_begin) that programs serve
+  // one record of kNarrowRecord ints per vnode of the narrow range, written by the host (or null):
+  // what a wave needs to start on the vnode in one memory round trip instead of two -- the vnode's
+  // four list entries, the requests of its rows and the pool slots of its first 32 tokens
+  const int32_t* narrow_table;
   int real_dim;                    // head dimension of the tensors; smaller than the kernel's D only for head_dim 16,
                                    // which the per-wave staging kernels compute as a zero-padded 32-dim contraction
   int g;
@@ -980,11 +984,20 @@ template <int D> struct NarrowGeom {
   static __device__ __forceinline__ int swz(int row) { return (((row & 3) << 2) | ((row >> 2) & 3)) & (kChunks - 1); }
 };
 
+// Layout of a narrow vnode's record in Stage1Args::narrow_table (ints): kv_off, kv_len, q_off,
+// q_len; then the requests of the vnode's first kNarrowRecRequests scratch rows; then the pool slots
+// of its first kTileTokens tokens (the last one repeated past the end of a shorter run).
+constexpr int kNarrowRecord = 64;
+constexpr int kNarrowRecRequests = 16;
+constexpr int kNarrowRecSlots = 4 + kNarrowRecRequests;
+
 // One wave's share of a narrow vnode for the 16 query rows from row0: the tiles tile0,
-// tile0 + tstride, ... of the run, staged in the wave's own LDS area at lds0.
+// tile0 + tstride, ... of the run, staged in the wave's own LDS area at lds0.  `rec` is the lane's
+// int of the vnode's record when `inlined` (else unused).
 template <typename E, int D, bool GATHERED>
 __device__ __forceinline__ void narrow_attend(const Stage1Args& a, const VnodeView& vn, char* smem, unsigned lds0,
-                                              int kvh, int row0, int tile0, int tstride, WaveState<D, 1>& st) {
+                                              int kvh, int row0, int tile0, int tstride, WaveState<D, 1>& st,
+                                              int rec = 0, bool inlined = false) {
   using N = NarrowGeom<D>;
   constexpr int KS = D / 32, DB = D / 16;
   constexpr float kSlackN = 8.f;
@@ -1013,10 +1026,16 @@ __device__ __forceinline__ void narrow_attend(const Stage1Args& a, const VnodeVi
   // start-up chain: [request id of the lane's row, slot indices] -> [Q fragments, first K/V rows].
   // Fragment ks of a lane: row row0 + p, dims 32*ks + 8*c .. +7; zero past the vnode.
   const char* q_src = nullptr;
-  if (row0 + p < vn.q_len * a.g) {
-    const int r = row0 + p, ri = r / a.g, rj = r - ri * a.g;
-    const int64_t entry = GATHERED ? (int64_t)(vn.q_off / a.nsplit) : (int64_t)a.q_entries[vn.q_off + ri];
-    q_src = a.q + 2 * (entry * a.sq0 + (int64_t)(kvh * a.g + rj) * a.sq1 + 8 * c);
+  {
+    const int r = min(row0 + p, max(vn.q_len * a.g - 1, 0)), ri = r / a.g, rj = r - ri * a.g;
+    // (the record holds the requests of the first rows; every lane takes part in the exchange)
+    const bool from_record = inlined && vn.q_len <= kNarrowRecRequests;
+    const int listed = from_record ? __shfl(rec, 4 + ri) : 0;
+    if (row0 + p < vn.q_len * a.g) {
+      const int64_t entry = GATHERED ? (int64_t)(vn.q_off / a.nsplit)
+                                     : (from_record ? (int64_t)listed : (int64_t)a.q_entries[vn.q_off + ri]);
+      q_src = a.q + 2 * (entry * a.sq0 + (int64_t)(kvh * a.g + rj) * a.sq1 + 8 * c);
+    }
   }
   u32x4 qf[1][KS];
   reset_state<D, 1>(st);
@@ -1058,9 +1077,27 @@ __device__ __forceinline__ void narrow_attend(const Stage1Args& a, const VnodeVi
         load_direct16(src, tile0_addr + (is_v ? N::kBytesK : 0) + g * 1024);
       }
     };
-    stage_indices(tile0 * kTileTokens);
-    issue(tile0, false);
-    issue(tile0, true);
+    // With the vnode's record at hand and the run's first tile to serve, the first 32 slot
+    // indices are already here: the rows are requested at once, and the rest of the window (if
+    // the run is longer than a tile) arrives beside them.
+    const bool from_record = !GATHERED && inlined && tile0 == 0;
+    int rest[N::kIdxCap / kWave];
+    if (from_record) {
+      if (lane >= kNarrowRecSlots && lane < kNarrowRecSlots + kTileTokens) idx_lds[lane - kNarrowRecSlots] = rec;
+      wave_lds_fence();
+      idx_base = 0;
+      issue(0, false);
+      issue(0, true);
+      if (vn.kv_len > kTileTokens) {
+#pragma unroll
+        for (int i = 0; i < N::kIdxCap / kWave; ++i)
+          rest[i] = a.kv_entries[vn.kv_base + min(kWave * i + lane, vn.kv_len - 1)];
+      }
+    } else {
+      stage_indices(tile0 * kTileTokens);
+      issue(tile0, false);
+      issue(tile0, true);
+    }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       u32x4 z = {0u, 0u, 0u, 0u};
@@ -1069,6 +1106,12 @@ __device__ __forceinline__ void narrow_attend(const Stage1Args& a, const VnodeVi
     // nothing the compiler itself tracks may still be in flight below: a wait for it would
     // also wait for every direct load
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    if (from_record && vn.kv_len > kTileTokens) {
+      // (the first tile's rows were requested with the record's indices, which these repeat)
+#pragma unroll
+      for (int i = 0; i < N::kIdxCap / kWave; ++i) idx_lds[kWave * i + lane] = rest[i];
+      wave_lds_fence();
+    }
     // (and the compiler must see the fragments as complete, or it keeps a wait for them in the loop)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[0][ks]));
@@ -1187,12 +1230,22 @@ __device__ __forceinline__ void narrow_item(const Stage1Args& a, char* smem, int
   using N = NarrowGeom<D>;
   const unsigned lds0 = (unsigned)slot * N::kLds;  // byte offset of the wave's area in the block's LDS segment
   VnodeView vn{0, 0, 0, 0};
-  if (exists) vn = load_vnode<GATHERED>(a, vnode);
+  int rec = 0;
+  const bool inlined = !GATHERED && a.narrow_table != nullptr;   // launch uniform
+  if (inlined) {
+    if (exists) rec = a.narrow_table[(int64_t)(vnode - a.narrow_begin) * kNarrowRecord + (threadIdx.x & 63)];
+    vn.kv_base = __builtin_amdgcn_readlane(rec, 0);
+    vn.kv_len = __builtin_amdgcn_readlane(rec, 1);
+    vn.q_off = __builtin_amdgcn_readlane(rec, 2);
+    vn.q_len = __builtin_amdgcn_readlane(rec, 3);
+  } else if (exists) {
+    vn = load_vnode<GATHERED>(a, vnode);
+  }
   const int rows_total = vn.q_len * a.g;
   if (share == 1) {
     for (int row0 = 0; row0 < rows_total; row0 += 16) {
       WaveState<D, 1> st;
-      narrow_attend<E, D, GATHERED>(a, vn, smem, lds0, kvh, row0, 0, 1, st);
+      narrow_attend<E, D, GATHERED>(a, vn, smem, lds0, kvh, row0, 0, 1, st, rec, inlined);
       write_partials<D, 1>(a, vn, kvh, row0, st);
     }
     return;
@@ -1210,7 +1263,7 @@ __device__ __forceinline__ void narrow_item(const Stage1Args& a, char* smem, int
   for (int pass = 0; pass < passes; ++pass) {
     const int row0 = 16 * pass;
     WaveState<D, 1> st;
-    if (row0 < rows_total) narrow_attend<E, D, GATHERED>(a, vn, smem, lds0, kvh, row0, w, share, st);
+    if (row0 < rows_total) narrow_attend<E, D, GATHERED>(a, vn, smem, lds0, kvh, row0, w, share, st, rec, inlined);
     else reset_state<D, 1>(st);
     merge_shares<D>(xchg, st, w, share);
     if (w == 0 && row0 < rows_total) write_partials<D, 1>(a, vn, kvh, row0, st);
@@ -2055,6 +2108,7 @@ int ft_stage1_programs(const void* q, const void* k, const void* v,
                        float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
                        const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
                        const int32_t* prog_table, int num_programs, int narrow_in_programs,
+                       const int32_t* narrow_table,
                        int num_qo_heads, int num_kv_heads, int head_dim,
                        float sm_scale, int dtype, ft_stream_t stream) {
   if (!phase_node_nums || !phase_node_offsets) return FT_ERR_NULL_POINTER;
@@ -2077,6 +2131,7 @@ int ft_stage1_programs(const void* q, const void* k, const void* v,
   a.vnode_begin = phase_node_offsets[0]; a.vnode_count = phase_node_nums[0];
   a.narrow_begin = phase_node_offsets[1]; a.narrow_count = phase_node_nums[1];
   if (num_programs > 0) { a.prog_table = prog_table; a.num_programs = num_programs; a.narrow_in_programs = narrow_in_programs; }
+  a.narrow_table = narrow_table;
   a.wide_rows = kWideRows;
   return launch_stage1<false>(a, head_dim, dtype, stream);
 }
@@ -2092,12 +2147,14 @@ int ft_decode_programs(const void* q, const void* k, const void* v, void* o,
                        float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
                        const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
                        const int32_t* prog_table, int num_programs, int narrow_in_programs,
+                       const int32_t* narrow_table,
                        int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
                        float sm_scale, int dtype, ft_stream_t stream) {
   if (int rc = ft_stage1_programs(q, k, v, sq0, sq1, sk0, sk1, sv0, sv1, vnode_to_kv_entries, vnode_to_kv_offs,
                                   vnode_to_kv_lens, vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, mid_o, so0,
                                   so1, mid_lse, sl0, phase_node_nums, phase_node_offsets, prog_table, num_programs,
-                                  narrow_in_programs, num_qo_heads, num_kv_heads, head_dim, sm_scale, dtype, stream))
+                                  narrow_in_programs, narrow_table, num_qo_heads, num_kv_heads, head_dim, sm_scale, dtype,
+                                  stream))
     return rc;
   return ft_stage2(req_to_vnode_entries, req_to_vnode_offs, req_to_vnode_lens, mid_o, so0, so1, mid_lse, sl0, o, oo0,
                    oo1, batch_size, num_qo_heads, head_dim, dtype, stream);
@@ -2113,6 +2170,7 @@ int ft_decode_static(const void* q, const void* k, const void* v, void* o,
                      const int32_t* req_to_vnode_lens, int64_t num_rows,
                      const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
                      const int32_t* prog_table, int num_programs, int narrow_in_programs,
+                     const int32_t* narrow_table,
                      int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
                      float sm_scale, int dtype, ft_stream_t stream) {
   if (num_rows < 0 || num_qo_heads < 1 || head_dim < 1) return FT_ERR_ARGUMENT;
@@ -2129,7 +2187,8 @@ int ft_decode_static(const void* q, const void* k, const void* v, void* o,
                             vnode_to_kv_lens, vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, req_to_vnode_entries,
                             req_to_vnode_offs, req_to_vnode_lens, mid_o, (int64_t)num_qo_heads * head_dim, head_dim,
                             mid_lse, num_qo_heads, phase_node_nums, phase_node_offsets, prog_table, num_programs,
-                            narrow_in_programs, batch_size, num_qo_heads, num_kv_heads, head_dim, sm_scale, dtype, stream);
+                            narrow_in_programs, narrow_table, batch_size, num_qo_heads, num_kv_heads, head_dim, sm_scale,
+                            dtype, stream);
 }
 
 int ft_decode(const void* q, const void* k, const void* v, void* o,

@@ -26,6 +26,12 @@ def _stream_handle(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+def _narrow_table_ptr(phase_node_nums):
+    """Device pointer of the narrow vnodes' records a launch-order plan carries, or None."""
+    table = getattr(phase_node_nums, "narrow_table", None)
+    return table.data_ptr() if table is not None else None
+
+
 def _need_gpu(*tensors):
     for t in tensors:
         if not t.is_cuda:
@@ -68,7 +74,8 @@ def fasttree_decode(
         raise _lib.FastTreeLibraryError("mid_o and mid_lse must be float32")
     lib = _lib.load()
     programs = getattr(phase_node_nums, "prog_table", None)
-    if programs is not None and q.shape[-1] >= 32:
+    narrow_table = _narrow_table_ptr(phase_node_nums)
+    if (programs is not None or narrow_table is not None) and q.shape[-1] >= 32:
         # the launch was arranged as block programs (launch_schedule.block_programs)
         rc = lib.ft_decode_programs(
             q.data_ptr(), k_buffer.data_ptr(), v_buffer.data_ptr(), o.data_ptr(),
@@ -79,7 +86,9 @@ def fasttree_decode(
             req_to_vnode_entries.data_ptr(), req_to_vnode_offs.data_ptr(), req_to_vnode_lens.data_ptr(),
             mid_o.data_ptr(), mid_o.stride(0), mid_o.stride(1), mid_lse.data_ptr(), mid_lse.stride(0),
             _lib.int32_pair(phase_node_nums), _lib.int32_pair(phase_node_offsets),
-            programs.data_ptr(), int(phase_node_nums.num_programs), int(phase_node_nums.narrow_in_programs),
+            programs.data_ptr() if programs is not None else None,
+            int(phase_node_nums.num_programs) if programs is not None else 0,
+            int(phase_node_nums.narrow_in_programs) if programs is not None else 0, narrow_table,
             q.shape[0], q.shape[1], k_buffer.shape[1], q.shape[-1],
             float(sm_scale), _dtype_code(q), _stream_handle(q),
         )
@@ -132,7 +141,9 @@ def fasttree_decode_static(q, k_buffer, v_buffer, o, vnode_to_kv_entries, vnode_
         int(vnode_to_q_entries.numel()),
         _lib.int32_pair(phase_node_nums), _lib.int32_pair(phase_node_offsets),
         programs.data_ptr() if programs is not None else None,
-        int(getattr(phase_node_nums, "num_programs", 0)), int(getattr(phase_node_nums, "narrow_in_programs", 0)),
+        int(getattr(phase_node_nums, "num_programs", 0)) if programs is not None else 0,
+        int(getattr(phase_node_nums, "narrow_in_programs", 0)) if programs is not None else 0,
+        _narrow_table_ptr(phase_node_nums),
         q.shape[0], q.shape[1], k_buffer.shape[1], q.shape[-1],
         float(sm_scale), _dtype_code(q), _stream_handle(q),
     )
@@ -147,7 +158,8 @@ def fasttree_decode_stage1(q, k_buffer, v_buffer, vnode_to_kv_entries, vnode_to_
     _need_gpu(q, k_buffer, v_buffer, mid_o, mid_lse)
     lib = _lib.load()
     programs = getattr(phase_node_nums, "prog_table", None)
-    if programs is not None and q.shape[-1] >= 32:
+    narrow_table = _narrow_table_ptr(phase_node_nums)
+    if (programs is not None or narrow_table is not None) and q.shape[-1] >= 32:
         rc = lib.ft_stage1_programs(
             q.data_ptr(), k_buffer.data_ptr(), v_buffer.data_ptr(),
             q.stride(0), q.stride(1), k_buffer.stride(0), k_buffer.stride(1), v_buffer.stride(0), v_buffer.stride(1),
@@ -155,7 +167,9 @@ def fasttree_decode_stage1(q, k_buffer, v_buffer, vnode_to_kv_entries, vnode_to_
             vnode_to_q_entries.data_ptr(), vnode_to_q_offs.data_ptr(), vnode_to_q_lens.data_ptr(),
             mid_o.data_ptr(), mid_o.stride(0), mid_o.stride(1), mid_lse.data_ptr(), mid_lse.stride(0),
             _lib.int32_pair(phase_node_nums), _lib.int32_pair(phase_node_offsets),
-            programs.data_ptr(), int(phase_node_nums.num_programs), int(phase_node_nums.narrow_in_programs),
+            programs.data_ptr() if programs is not None else None,
+            int(phase_node_nums.num_programs) if programs is not None else 0,
+            int(phase_node_nums.narrow_in_programs) if programs is not None else 0, narrow_table,
             q.shape[1], k_buffer.shape[1], q.shape[-1], float(sm_scale), _dtype_code(q), _stream_handle(q),
         )
         _lib.check(rc, "ft_stage1_programs")

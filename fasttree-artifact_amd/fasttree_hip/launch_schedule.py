@@ -142,6 +142,8 @@ class LaunchPhases(list):
     prog_table = None
     num_programs = 0
     narrow_in_programs = 0
+    #: int32 device tensor of :func:`narrow_records` (64 entries per vnode of the second phase), or None
+    narrow_table = None
     #: what the schedule's model expects the first-stage launch to take, and the machine it was laid out for
     modelled_us = None
     num_cus = None
@@ -174,6 +176,40 @@ class LaunchSchedule:
     @property
     def num_programs(self) -> int:
         return int(self.prog_table.shape[0])
+
+
+#: Whether launch-order plans carry the records of :func:`narrow_records` (a switch for measurements).
+USE_NARROW_RECORDS = True
+#: Entries of a narrow vnode's record, requests and token slots it holds (the kernels' layout).
+NARROW_RECORD = 64
+NARROW_RECORD_REQUESTS = 16
+NARROW_RECORD_TOKENS = 32
+
+
+def narrow_records(kv_entries, kv_offs, kv_lens, q_offs, q_lens, q_entries, first, count):
+    """One record per vnode ``first .. first + count - 1`` of the lists (the narrow phase): what a
+    wave needs to start on the vnode, in one place, so that it finds it in one memory round trip
+    instead of two (the vnode's four list entries, then its slot indices and requests) before it
+    can ask for K/V rows.  Entries: ``kv_off, kv_len, q_off, q_len``, the requests of the first 16
+    scratch rows, the pool slots of the first 32 tokens (the last token repeated past the end of a
+    shorter run), padding.  Returns an int32 array ``[count, 64]``."""
+    kv_entries = np.asarray(kv_entries).reshape(-1)
+    q_entries = np.asarray(q_entries).reshape(-1)
+    table = np.zeros((int(count), NARROW_RECORD), dtype=np.int32)
+    if count == 0:
+        return table
+    sl = slice(int(first), int(first) + int(count))
+    ko, kl = np.asarray(kv_offs[sl], dtype=np.int64), np.asarray(kv_lens[sl], dtype=np.int64)
+    qo, ql = np.asarray(q_offs[sl], dtype=np.int64), np.asarray(q_lens[sl], dtype=np.int64)
+    table[:, 0], table[:, 1], table[:, 2], table[:, 3] = ko, kl, qo, ql
+    rows = qo[:, None] + np.minimum(np.arange(NARROW_RECORD_REQUESTS)[None, :], np.maximum(ql[:, None] - 1, 0))
+    table[:, 4:4 + NARROW_RECORD_REQUESTS] = np.where(ql[:, None] > 0, q_entries[np.minimum(rows, max(len(q_entries) - 1, 0))], 0) \
+        if len(q_entries) else 0
+    tokens = ko[:, None] + np.minimum(np.arange(NARROW_RECORD_TOKENS)[None, :], np.maximum(kl[:, None] - 1, 0))
+    first_slot = 4 + NARROW_RECORD_REQUESTS
+    table[:, first_slot:first_slot + NARROW_RECORD_TOKENS] = np.where(
+        kl[:, None] > 0, kv_entries[np.minimum(tokens, max(len(kv_entries) - 1, 0))], 0) if len(kv_entries) else 0
+    return table
 
 
 _CUS_OF_DEVICE = {}

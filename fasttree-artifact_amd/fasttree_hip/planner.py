@@ -447,6 +447,7 @@ class PlanBuffers:
         self.req_to_vnode_entries = ints(max_rows + 32)
         self.req_to_vnode_offs, self.req_to_vnode_lens = ints(max_batch_size), ints(max_batch_size)
         self.prog_table = ints(4 * max_vnodes)
+        self.narrow_table = ints(64 * max_vnodes)     # (launch_schedule.NARROW_RECORD entries per narrow vnode)
         self.mid_o = torch.empty((int(max_rows), num_qo_heads, head_dim), dtype=torch.float32, device=device)
         self.mid_lse = torch.empty((int(max_rows), num_qo_heads), dtype=torch.float32, device=device)
 
@@ -541,6 +542,11 @@ def fasttree_preparation(
             phase_nums.prog_table = place("prog_table", sched.prog_table.reshape(-1))
             phase_nums.num_programs = sched.num_programs
             phase_nums.narrow_in_programs = sched.narrow_in_programs
+        from . import launch_schedule
+        if phase_nums[1] > 0 and head_dim >= 32 and launch_schedule.USE_NARROW_RECORDS:
+            from .launch_schedule import narrow_records
+            records = narrow_records(plan.vnode_to_kv_entries, *vnodes, q_entries, phase_offs[1], phase_nums[1])
+            phase_nums.narrow_table = place("narrow_table", records.reshape(-1))
     if buffers is not None:
         if rows > buffers.mid_o.shape[0] or buffers.mid_o.shape[1:] != (num_qo_heads, head_dim):
             raise ValueError(f"the scratch of the buffers ({tuple(buffers.mid_o.shape)}) does not hold "

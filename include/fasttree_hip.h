@@ -133,6 +133,14 @@ int ft_decode(const void* q, const void* k, const void* v, void* o,
  * ft_stage1_phases, whatever their width.  The lists are otherwise those of ft_decode and
  * describe a complete plan without the table.  head_dim in {32, 64, 128, 256}.  The table is
  * trusted: it is not read on the host.
+ *
+ * narrow_table (or NULL) holds one record of 64 int32 per vnode of the second range, in the range's
+ * order: the vnode's kv_off, kv_len, q_off and q_len as in the lists; then the requests of its first
+ * 16 scratch rows (vnode_to_q_entries[q_off ...], unused entries anything); then the pool slots of its
+ * first 32 tokens (vnode_to_kv_entries[kv_off + min(t, kv_len - 1)]); the rest is padding.  A wave that
+ * serves such a vnode then starts with one memory round trip (the record) instead of two (the four
+ * list entries, then the index and request lists) before it can ask for K/V rows.  The records must
+ * agree with the lists; they are trusted like them.
  */
 int ft_stage1_programs(const void* q, const void* k, const void* v,
                        int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
@@ -142,6 +150,7 @@ int ft_stage1_programs(const void* q, const void* k, const void* v,
                        float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
                        const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
                        const int32_t* prog_table, int num_programs, int narrow_in_programs,
+                       const int32_t* narrow_table,
                        int num_qo_heads, int num_kv_heads, int head_dim,
                        float sm_scale, int dtype, ft_stream_t stream);
 
@@ -156,6 +165,7 @@ int ft_decode_programs(const void* q, const void* k, const void* v, void* o,
                        float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
                        const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
                        const int32_t* prog_table, int num_programs, int narrow_in_programs,
+                       const int32_t* narrow_table,
                        int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
                        float sm_scale, int dtype, ft_stream_t stream);
 
@@ -196,6 +206,7 @@ int ft_decode_static(const void* q, const void* k, const void* v, void* o,
                      const int32_t* req_to_vnode_lens, int64_t num_rows,
                      const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
                      const int32_t* prog_table, int num_programs, int narrow_in_programs,
+                     const int32_t* narrow_table,
                      int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
                      float sm_scale, int dtype, ft_stream_t stream);
 

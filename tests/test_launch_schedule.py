@@ -273,3 +273,40 @@ def test_fewer_compute_units_mean_fewer_and_longer_programs():
     assert small.modelled_us > full.modelled_us >= large.modelled_us
     # without a device to ask, the default machine is an MI355X's 256 units
     assert ls.compute_units("cpu") == 256 == ls.DEFAULT_COMPUTE_UNITS
+
+
+def test_narrow_records_repeat_the_lists():
+    """The record of a narrow vnode holds what the lists say about it: its four entries, the
+    requests of its scratch rows and the pool slots of its first 32 tokens, the last one repeated
+    past the end of a shorter run (hand case, then every narrow vnode of two launch-order plans)."""
+    kv_entries = np.arange(1000, 1100)
+    rec = ls.narrow_records(kv_entries, [0, 10, 50], [10, 40, 3], [0, 2, 3], [2, 1, 4], [7, 8, 9, 3, 4, 5, 6], 1, 2)
+    assert rec.shape == (2, 64) and rec.dtype == np.int32
+    assert rec[0, :4].tolist() == [10, 40, 2, 1] and rec[0, 4] == 9
+    assert rec[0, 20:52].tolist() == list(range(1010, 1042))
+    assert rec[1, :4].tolist() == [50, 3, 3, 4] and rec[1, 4:8].tolist() == [3, 4, 5, 6]
+    assert rec[1, 20:52].tolist() == [1050, 1051] + [1052] * 30
+    assert ls.narrow_records(kv_entries, [0], [0], [0], [0], [], 0, 1)[0].tolist() == [0] * 64     # an empty vnode
+    import torch
+    from fasttree_hip.planner import FastTreeParams, fasttree_preparation
+    import fasttree_hip.planner as planner_module
+    planner_module.VERBOSE = False
+    for name in ("c3", "c5_seed0", "c1"):
+        case = next(c for c in PLANNER_CASES if c["name"] == name)
+        tree, ptrs, batch = build_tree(case["tree"])
+        g = case["Hq"] // case["Hkv"]
+        p = FastTreeParams(); p.set_values(0.66, 0.33, 0.1); p.set_q_tile_sizes([max(1, 64 // g), max(1, 16 // g)])
+        p.set_kv_tile_sizes([32, 32]); p.set_kv_group_num(g)
+        slot_map = np.random.default_rng(0).permutation(ptrs[-1])
+        aux, _ = fasttree_preparation(tree, ptrs, batch, case["Hq"], case["Hkv"], 128, [1024, 256], [256, 1024], [256, 256], p,
+                                      device="cpu", kv_slot_map=slot_map, launch_order=True)
+        nums, offs = aux[11], aux[12]
+        table = nums.narrow_table.view(-1, 64).numpy()
+        assert table.shape[0] == nums[1] > 0
+        kv_entries, kv_offs, kv_lens, q_entries, q_offs, q_lens = (t.numpy() for t in aux[:6])
+        for i in range(0, nums[1], max(1, nums[1] // 50)):
+            v = offs[1] + i
+            assert table[i, :4].tolist() == [kv_offs[v], kv_lens[v], q_offs[v], q_lens[v]]
+            assert table[i, 4:4 + min(q_lens[v], 16)].tolist() == q_entries[q_offs[v]: q_offs[v] + min(q_lens[v], 16)].tolist()
+            want = [kv_entries[kv_offs[v] + min(t, kv_lens[v] - 1)] for t in range(32)]
+            assert table[i, 20:52].tolist() == want
