@@ -275,7 +275,7 @@ def test_fewer_compute_units_mean_fewer_and_longer_programs():
     assert ls.compute_units("cpu") == 256 == ls.DEFAULT_COMPUTE_UNITS
 
 
-def test_narrow_records_repeat_the_lists():
+def test_narrow_records_repeat_the_lists(monkeypatch):
     """The record of a narrow vnode holds what the lists say about it: its four entries, the
     requests of its scratch rows and the pool slots of its first 32 tokens, the last one repeated
     past the end of a shorter run (hand case, then every narrow vnode of two launch-order plans)."""
@@ -290,7 +290,7 @@ def test_narrow_records_repeat_the_lists():
     import torch
     from fasttree_hip.planner import FastTreeParams, fasttree_preparation
     import fasttree_hip.planner as planner_module
-    planner_module.VERBOSE = False
+    monkeypatch.setattr(planner_module, "VERBOSE", False)
     for name in ("c3", "c5_seed0", "c1"):
         case = next(c for c in PLANNER_CASES if c["name"] == name)
         tree, ptrs, batch = build_tree(case["tree"])
