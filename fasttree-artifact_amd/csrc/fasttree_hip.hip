@@ -1584,7 +1584,13 @@ struct Stage2Args {
   int64_t oo0, oo1;
   int batch, hq;
   int nsplit;  // > 0: gathered mode, request r owns rows [r*nsplit, (r+1)*nsplit)
+  // (or null) one record of kReqRecord int32 per request, written by the host: req_lens[r],
+  // req_offs[r], then the request's first kReqRecord - 2 entries -- what the block needs before
+  // it can ask for the partial rows, in one memory round trip instead of two
+  const int32_t* req_table;
 };
+constexpr int kReqRecord = 16;
+constexpr int kReqRecEntries = kReqRecord - 2;
 
 template <int WIDTH> __device__ __forceinline__ float group_max(float x) {
 #pragma unroll
@@ -1609,15 +1615,30 @@ __global__ void __launch_bounds__(kBlock) stage2_kernel(Stage2Args a) {
   const int req = blockIdx.x;
   const int head = blockIdx.y * HPB + grp;
   if (head >= a.hq) return;
-  const int off = a.nsplit > 0 ? req * a.nsplit : a.req_offs[req];
-  const int n = a.nsplit > 0 ? a.nsplit : a.req_lens[req];
+  const int32_t* rec = a.req_table ? a.req_table + (int64_t)req * kReqRecord : nullptr;  // launch uniform
+  int off, n, rec_row = -1;
+  if (a.nsplit > 0) {
+    off = req * a.nsplit;
+    n = a.nsplit;
+  } else if (rec) {
+    n = rec[0];
+    off = rec[1];
+    rec_row = rec[2 + min(gl, kReqRecEntries - 1)];  // (requested together with the two words above)
+  } else {
+    off = a.req_offs[req];
+    n = a.req_lens[req];
+  }
 
   float m_run = -INFINITY, l_run = 0.f;
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   for (int base = 0; base < n; base += LPH) {
     const int cnt = min(LPH, n - base);
     int my_row = -1;
-    if (gl < cnt) my_row = a.nsplit > 0 ? off + base + gl : a.req_entries[off + base + gl];
+    if (gl < cnt) {
+      if (a.nsplit > 0) my_row = off + base + gl;
+      else if (rec && base + gl < kReqRecEntries) my_row = base == 0 ? rec_row : rec[2 + base + gl];
+      else my_row = a.req_entries[off + base + gl];
+    }
     // Rows in batches of kBatch, all loads of a batch issued before the first is used (the rows
     // are in bounds whatever their weight; a zero weight discards the row's contents).  The
     // first batch is requested together with the log-sum-exp values, not after them: both
@@ -2029,11 +2050,11 @@ int ft_stage1(const void* q, const void* k, const void* v,
   return launch_stage1<false>(a, head_dim, dtype, stream);
 }
 
-int ft_stage2(const int32_t* req_to_vnode_entries, const int32_t* req_to_vnode_offs,
-              const int32_t* req_to_vnode_lens,
-              const float* mid_o, int64_t so0, int64_t so1, const float* mid_lse, int64_t sl0,
-              void* o, int64_t oo0, int64_t oo1,
-              int batch_size, int num_qo_heads, int head_dim, int dtype, ft_stream_t stream) {
+static int stage2_with_table(const int32_t* req_to_vnode_entries, const int32_t* req_to_vnode_offs,
+                             const int32_t* req_to_vnode_lens, const int32_t* req_table,
+                             const float* mid_o, int64_t so0, int64_t so1, const float* mid_lse, int64_t sl0,
+                             void* o, int64_t oo0, int64_t oo1,
+                             int batch_size, int num_qo_heads, int head_dim, int dtype, ft_stream_t stream) {
   if (int rc = check_common(head_dim, 1, dtype)) return rc;
   if (batch_size == 0) return FT_OK;
   if (!req_to_vnode_entries || !req_to_vnode_offs || !req_to_vnode_lens || !mid_o || !mid_lse || !o)
@@ -2045,7 +2066,17 @@ int ft_stage2(const int32_t* req_to_vnode_entries, const int32_t* req_to_vnode_o
   a.mid_o = mid_o; a.so0 = so0; a.so1 = so1; a.mid_lse = mid_lse; a.sl0 = sl0;
   a.o = static_cast<char*>(o); a.oo0 = oo0; a.oo1 = oo1;
   a.batch = batch_size; a.hq = num_qo_heads; a.nsplit = 0;
+  a.req_table = req_table;
   return launch_stage2(a, head_dim, dtype, stream);
+}
+
+int ft_stage2(const int32_t* req_to_vnode_entries, const int32_t* req_to_vnode_offs,
+              const int32_t* req_to_vnode_lens,
+              const float* mid_o, int64_t so0, int64_t so1, const float* mid_lse, int64_t sl0,
+              void* o, int64_t oo0, int64_t oo1,
+              int batch_size, int num_qo_heads, int head_dim, int dtype, ft_stream_t stream) {
+  return stage2_with_table(req_to_vnode_entries, req_to_vnode_offs, req_to_vnode_lens, nullptr, mid_o, so0, so1, mid_lse,
+                           sl0, o, oo0, oo1, batch_size, num_qo_heads, head_dim, dtype, stream);
 }
 
 int ft_stage1_phases(const void* q, const void* k, const void* v,
@@ -2147,7 +2178,7 @@ int ft_decode_programs(const void* q, const void* k, const void* v, void* o,
                        float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
                        const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
                        const int32_t* prog_table, int num_programs, int narrow_in_programs,
-                       const int32_t* narrow_table,
+                       const int32_t* narrow_table, const int32_t* req_table,
                        int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
                        float sm_scale, int dtype, ft_stream_t stream) {
   if (int rc = ft_stage1_programs(q, k, v, sq0, sq1, sk0, sk1, sv0, sv1, vnode_to_kv_entries, vnode_to_kv_offs,
@@ -2156,8 +2187,8 @@ int ft_decode_programs(const void* q, const void* k, const void* v, void* o,
                                   narrow_in_programs, narrow_table, num_qo_heads, num_kv_heads, head_dim, sm_scale, dtype,
                                   stream))
     return rc;
-  return ft_stage2(req_to_vnode_entries, req_to_vnode_offs, req_to_vnode_lens, mid_o, so0, so1, mid_lse, sl0, o, oo0,
-                   oo1, batch_size, num_qo_heads, head_dim, dtype, stream);
+  return stage2_with_table(req_to_vnode_entries, req_to_vnode_offs, req_to_vnode_lens, req_table, mid_o, so0, so1,
+                           mid_lse, sl0, o, oo0, oo1, batch_size, num_qo_heads, head_dim, dtype, stream);
 }
 
 int ft_decode_static(const void* q, const void* k, const void* v, void* o,
@@ -2170,7 +2201,7 @@ int ft_decode_static(const void* q, const void* k, const void* v, void* o,
                      const int32_t* req_to_vnode_lens, int64_t num_rows,
                      const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
                      const int32_t* prog_table, int num_programs, int narrow_in_programs,
-                     const int32_t* narrow_table,
+                     const int32_t* narrow_table, const int32_t* req_table,
                      int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
                      float sm_scale, int dtype, ft_stream_t stream) {
   if (num_rows < 0 || num_qo_heads < 1 || head_dim < 1) return FT_ERR_ARGUMENT;
@@ -2187,8 +2218,8 @@ int ft_decode_static(const void* q, const void* k, const void* v, void* o,
                             vnode_to_kv_lens, vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, req_to_vnode_entries,
                             req_to_vnode_offs, req_to_vnode_lens, mid_o, (int64_t)num_qo_heads * head_dim, head_dim,
                             mid_lse, num_qo_heads, phase_node_nums, phase_node_offsets, prog_table, num_programs,
-                            narrow_in_programs, narrow_table, batch_size, num_qo_heads, num_kv_heads, head_dim, sm_scale,
-                            dtype, stream);
+                            narrow_in_programs, narrow_table, req_table, batch_size, num_qo_heads, num_kv_heads, head_dim,
+                            sm_scale, dtype, stream);
 }
 
 int ft_decode(const void* q, const void* k, const void* v, void* o,

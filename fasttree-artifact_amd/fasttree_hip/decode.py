@@ -32,6 +32,12 @@ def _narrow_table_ptr(phase_node_nums):
     return table.data_ptr() if table is not None else None
 
 
+def _req_table_ptr(phase_node_nums):
+    """Device pointer of the per-request records for the merge launch, or None."""
+    table = getattr(phase_node_nums, "req_table", None)
+    return table.data_ptr() if table is not None else None
+
+
 def _need_gpu(*tensors):
     for t in tensors:
         if not t.is_cuda:
@@ -89,6 +95,7 @@ def fasttree_decode(
             programs.data_ptr() if programs is not None else None,
             int(phase_node_nums.num_programs) if programs is not None else 0,
             int(phase_node_nums.narrow_in_programs) if programs is not None else 0, narrow_table,
+            _req_table_ptr(phase_node_nums),
             q.shape[0], q.shape[1], k_buffer.shape[1], q.shape[-1],
             float(sm_scale), _dtype_code(q), _stream_handle(q),
         )
@@ -143,7 +150,7 @@ def fasttree_decode_static(q, k_buffer, v_buffer, o, vnode_to_kv_entries, vnode_
         programs.data_ptr() if programs is not None else None,
         int(getattr(phase_node_nums, "num_programs", 0)) if programs is not None else 0,
         int(getattr(phase_node_nums, "narrow_in_programs", 0)) if programs is not None else 0,
-        _narrow_table_ptr(phase_node_nums),
+        _narrow_table_ptr(phase_node_nums), _req_table_ptr(phase_node_nums),
         q.shape[0], q.shape[1], k_buffer.shape[1], q.shape[-1],
         float(sm_scale), _dtype_code(q), _stream_handle(q),
     )

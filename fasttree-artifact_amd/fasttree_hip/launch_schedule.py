@@ -73,6 +73,9 @@ VNODE_STARTUP_TILES = 5.0
 #: A narrow vnode on one wave, in the same unit: its start-up and one 32-token step.
 NARROW_STARTUP_TILES = 3.8
 NARROW_STEP_TILES = 0.85
+#: What the merge of the waves that share one narrow vnode costs each of them (two block barriers
+#: and an exchange of the state through LDS per halving), in the same unit.
+NARROW_SHARE_TILES = 0.5
 #: Microseconds per tile step of a block that shares its compute unit with another wide block,
 #: and of one that does not (measured on the 3-level tree of the headline benchmark).
 TILE_US_SHARED = 1.19
@@ -80,11 +83,11 @@ TILE_US_ALONE = 0.95
 #: Bytes per microsecond the narrow vnodes stream at most on DEFAULT_COMPUTE_UNITS units (rows of
 #: 2 * head_dim bytes at random slots); taken to scale with the number of units.
 NARROW_BYTES_PER_US = 5.6e6
-#: What a launch costs before its first block runs and after its last one ends, as seen between two
-#: events on the launch stream (measured on launches of a few vnodes: 15 us between events where the
-#: blocks themselves model at 12).  Part of the reported duration only: it is the same for every
-#: layout of a launch, so the choice between layouts does not see it.
-LAUNCH_US = 3.0
+#: What a launch costs on top of its blocks' own time when launches are queued back to back on one
+#: stream (measured: launches of 192 narrow vnodes, whose waves model at 5.5 us, repeat every 7.0 us).
+#: Part of the reported duration only: it is the same for every layout of a launch, so the choice
+#: between layouts does not see it.
+LAUNCH_US = 1.5
 #: A tile step of a piece of at most 64 query rows, relative to one of a full block.  The block's
 #: waves then split the tokens of a super tile, but the super tile is loaded all the same: fitted on
 #: the programs of an irregular tree of 500 requests, 1.21 against 1.44 us per tile step.
@@ -144,6 +147,8 @@ class LaunchPhases(list):
     narrow_in_programs = 0
     #: int32 device tensor of :func:`narrow_records` (64 entries per vnode of the second phase), or None
     narrow_table = None
+    #: int32 device tensor of :func:`request_records` (16 entries per request), or None
+    req_table = None
     #: what the schedule's model expects the first-stage launch to take, and the machine it was laid out for
     modelled_us = None
     num_cus = None
@@ -180,6 +185,8 @@ class LaunchSchedule:
 
 #: Whether launch-order plans carry the records of :func:`narrow_records` (a switch for measurements).
 USE_NARROW_RECORDS = True
+#: Whether they carry the records of :func:`request_records` for the merge launch (likewise).
+USE_REQUEST_RECORDS = True
 #: Entries of a narrow vnode's record, requests and token slots it holds (the kernels' layout).
 NARROW_RECORD = 64
 NARROW_RECORD_REQUESTS = 16
@@ -209,6 +216,31 @@ def narrow_records(kv_entries, kv_offs, kv_lens, q_offs, q_lens, q_entries, firs
     first_slot = 4 + NARROW_RECORD_REQUESTS
     table[:, first_slot:first_slot + NARROW_RECORD_TOKENS] = np.where(
         kl[:, None] > 0, kv_entries[np.minimum(tokens, max(len(kv_entries) - 1, 0))], 0) if len(kv_entries) else 0
+    return table
+
+
+#: Entries of one request's record for the second stage: its number of scratch rows, where they
+#: start in the per-request list, and the first REQUEST_RECORD - 2 of them.
+REQUEST_RECORD = 16
+
+
+def request_records(req_entries, req_offs, req_lens):
+    """One record per request for the merge launch: ``req_lens[r], req_offs[r]`` and the first 14
+    scratch rows of the request (zeros past its last), so that a block of that launch knows
+    which partial rows to ask for after one memory round trip instead of two (length and offset,
+    then the list).  Rows beyond the fourteenth are read from the list.  Returns an int32 array
+    ``[len(req_offs), 16]``."""
+    req_entries = np.asarray(req_entries).reshape(-1)
+    offs, lens = np.asarray(req_offs, dtype=np.int64).reshape(-1), np.asarray(req_lens, dtype=np.int64).reshape(-1)
+    table = np.zeros((len(offs), REQUEST_RECORD), dtype=np.int32)
+    if len(offs) == 0:
+        return table
+    table[:, 0], table[:, 1] = lens, offs
+    inside = REQUEST_RECORD - 2
+    pos = offs[:, None] + np.arange(inside)[None, :]
+    held = np.arange(inside)[None, :] < lens[:, None]
+    if len(req_entries):
+        table[:, 2:] = np.where(held, req_entries[np.minimum(pos, len(req_entries) - 1)], 0)
     return table
 
 
@@ -631,12 +663,22 @@ def _block_programs(runs, batch_size, group, num_kv_heads, *,
         narrow_first = sum(len(sh) for sh in shares)
         trailing = narrow[narrow_first:]
         if trailing:
-            item_us = [narrow_work(v) * TILE_US_SHARED for v in trailing]
-            narrow_bytes = sum(v[1] for v in trailing) * heads * 4 * head_dim
-            slots_for_narrow = wave_slots if shared or not programs else wave_slots // 2
+            # the kernel's launcher lets 2 or 4 waves share a vnode of the trailing blocks while that
+            # leaves a quarter of the wave slots free; each then walks its share of the tiles
+            items = sum(-(-len(v[2]) * group // NARROW_ROWS) for v in trailing) * heads
+            share = 1
+            while share < BLOCK_WAVES and 4 * items * 2 * share <= 3 * wave_slots:
+                share *= 2
 
-            def narrow_us(wave_slots):
-                return max(sum(item_us) * heads / wave_slots, max(item_us), narrow_bytes / (NARROW_BYTES_PER_US * num_cus / DEFAULT_COMPUTE_UNITS))
+            def item_work(v):
+                steps = -(-tiles(v[1]) // share) * -(-len(v[2]) * group // NARROW_ROWS)
+                return NARROW_STARTUP_TILES + NARROW_STEP_TILES * steps + (NARROW_SHARE_TILES if share > 1 else 0.0)
+
+            item_us = [item_work(v) * TILE_US_SHARED for v in trailing]
+            narrow_bytes = sum(v[1] for v in trailing) * heads * 4 * head_dim
+            # (a vnode holds `share` wave slots for as long as its waves walk their tiles)
+            narrow_all_slots = max(sum(item_us) * heads * share / wave_slots, max(item_us),
+                                   narrow_bytes / (NARROW_BYTES_PER_US * num_cus / DEFAULT_COMPUTE_UNITS))
 
             if overlap:
                 # unequal programs end one after the other and the trailing blocks take their slots
@@ -649,9 +691,13 @@ def _block_programs(runs, batch_size, group, num_kv_heads, *,
                 else:
                     longest_us = max(program_tiles) * tile_us
                 modelled = max(longest_us,
-                               sum(program_tiles) * heads / float(block_slots) * tile_us + narrow_us(wave_slots))
+                               sum(program_tiles) * heads / float(block_slots) * tile_us + narrow_all_slots)
+            elif shared or not programs:
+                modelled = wide_us + narrow_all_slots
             else:
-                modelled = wide_us + narrow_us(wave_slots) if shared else max(wide_us, narrow_us(slots_for_narrow))
+                # programs on one block slot of every unit: the trailing blocks have the other half of
+                # the wave slots while the programs run (and work at half their rate), all of them after
+                modelled = max(wide_us, narrow_all_slots + wide_us / 2.0, max(item_us))
         else:
             modelled = wide_us
 

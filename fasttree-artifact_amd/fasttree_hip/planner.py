@@ -448,6 +448,7 @@ class PlanBuffers:
         self.req_to_vnode_offs, self.req_to_vnode_lens = ints(max_batch_size), ints(max_batch_size)
         self.prog_table = ints(4 * max_vnodes)
         self.narrow_table = ints(64 * max_vnodes)     # (launch_schedule.NARROW_RECORD entries per narrow vnode)
+        self.req_table = ints(16 * max_batch_size)    # (launch_schedule.REQUEST_RECORD entries per request)
         self.mid_o = torch.empty((int(max_rows), num_qo_heads, head_dim), dtype=torch.float32, device=device)
         self.mid_lse = torch.empty((int(max_rows), num_qo_heads), dtype=torch.float32, device=device)
 
@@ -547,6 +548,9 @@ def fasttree_preparation(
             from .launch_schedule import narrow_records
             records = narrow_records(plan.vnode_to_kv_entries, *vnodes, q_entries, phase_offs[1], phase_nums[1])
             phase_nums.narrow_table = place("narrow_table", records.reshape(-1))
+        if head_dim >= 32 and launch_schedule.USE_REQUEST_RECORDS:
+            from .launch_schedule import request_records
+            phase_nums.req_table = place("req_table", request_records(*per_request).reshape(-1))
     if buffers is not None:
         if rows > buffers.mid_o.shape[0] or buffers.mid_o.shape[1:] != (num_qo_heads, head_dim):
             raise ValueError(f"the scratch of the buffers ({tuple(buffers.mid_o.shape)}) does not hold "

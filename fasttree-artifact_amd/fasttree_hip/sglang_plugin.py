@@ -93,6 +93,8 @@ class FastTreeMetadata:
         self.mid_lse = torch.empty((max_vnode_to_q_entries, num_qo_heads), dtype=torch.float32, device=device)
         #: not in the reference: the block programs of a launch-order plan (four entries each)
         self.prog_table = ints(4 * max_vnodes)
+        #: not in the reference: a launch-order plan's record per request for the merge launch
+        self.req_table = ints(16 * max_batch_size)
 
         self.phase_node_nums: Optional[Sequence[int]] = None
         self.phase_node_offsets: Optional[Sequence[int]] = None
@@ -333,6 +335,7 @@ def prepare_for_fasttree_meta(batch, fasttree_metadata: FastTreeMetadata):
     lists = [[x[i] for i in perm] for x in (kv_offs, kv_lens, q_offs, q_lens)]
     meta.prog_table_len = 0
     if getattr(meta, "launch_order", False):
+        from . import launch_schedule
         from .launch_schedule import LaunchPhases, block_programs
 
         # the same computation as block programs: long shared runs (a system prompt
@@ -363,6 +366,10 @@ def prepare_for_fasttree_meta(batch, fasttree_metadata: FastTreeMetadata):
             nums.prog_table = meta.prog_table[: src.numel()]
             nums.num_programs = sched.num_programs
             nums.narrow_in_programs = sched.narrow_in_programs
+        if sched.num_programs > 0 and launch_schedule.USE_REQUEST_RECORDS and len(req_offs) * 16 <= meta.req_table.numel():
+            src = torch.from_numpy(launch_schedule.request_records(req_entries, req_offs, req_lens).reshape(-1))
+            meta.req_table[: src.numel()].copy_(src, non_blocking=True)
+            nums.req_table = meta.req_table[: src.numel()]
         meta.phase_node_nums, meta.phase_node_offsets = nums, list(sched.phase_node_offsets)
 
     def upload(dst, values):

@@ -168,21 +168,31 @@ def main(args):
         modelled = getattr(fasttree_aux[11], "modelled_us", None)
         if modelled is not None and not args.signature:
             # what the launch schedule's model expects of the first-stage launch beside what it takes: the
-            # median over back-to-back launches (warm caches, as the model's constants were measured)
+            # launches run back to back behind a filler that keeps the device busy while the host queues them
+            # (so the host's call rate and the cost of an event between two launches stay out of the figure;
+            # warm caches, as the model's constants were measured), timed in runs of twenty
             def call_stage1():
                 fasttree_decode_stage1(Q, K_tree_tensor, V_tree_tensor, *fasttree_aux[:6], sm_scale, fasttree_aux[9],
                                        fasttree_aux[10], fasttree_aux[11], fasttree_aux[12], q_tiles, kv_tiles)
 
             for _ in range(20):
                 call_stage1()
-            marks = [torch.cuda.Event(enable_timing=True) for _ in range(61)]
-            marks[0].record()
-            for i in range(60):
+            filler = torch.empty(int(256e6), dtype=torch.int8, device="cuda")
+            runs, per_run = 5, 20
+            marks = [torch.cuda.Event(enable_timing=True) for _ in range(runs + 1)]
+            torch.cuda.synchronize()
+            for _ in range(32):
+                filler.zero_()
+            for _ in range(per_run):                    # (these also write the filler's dirty lines back)
                 call_stage1()
+            marks[0].record()
+            for i in range(runs):
+                for _ in range(per_run):
+                    call_stage1()
                 marks[i + 1].record()
             torch.cuda.synchronize()
-            measured = torch.tensor([a.elapsed_time(b) for a, b in zip(marks, marks[1:])]).median().item() * 1e3
-            print(f"fasttree stage 1: modelled {modelled:.1f} us, measured {measured:.1f} us between events (warm), "
+            measured = torch.tensor([a.elapsed_time(b) for a, b in zip(marks, marks[1:])]).median().item() * 1e3 / per_run
+            print(f"fasttree stage 1: modelled {modelled:.1f} us, measured {measured:.1f} us per launch back to back (warm), "
                   f"{fasttree_aux[11].num_programs} programs on {fasttree_aux[11].block_slots} block slots", flush=True)
             results["stage1_modelled_us"], results["stage1_measured_us"] = float(modelled), float(measured)
 

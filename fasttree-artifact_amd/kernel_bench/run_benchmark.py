@@ -126,7 +126,7 @@ def write_table(rows, path):
 
 def write_model_check(rows, path):
     """The launch schedule's modelled duration of the first-stage launch beside the measured one
-    (warm, between events on the launch stream: the kernel plus 2-4 us of launch gap), for the
+    (warm, per launch of a run of launches queued back to back: the kernel plus the gap before the next one), for the
     cases whose lists were arranged as block programs."""
     rows = [r for r in rows if r.get("modelled_us") is not None]
     with open(path, "w") as fh:

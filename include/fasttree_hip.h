@@ -141,6 +141,13 @@ int ft_decode(const void* q, const void* k, const void* v, void* o,
  * serves such a vnode then starts with one memory round trip (the record) instead of two (the four
  * list entries, then the index and request lists) before it can ask for K/V rows.  The records must
  * agree with the lists; they are trusted like them.
+ *
+ * req_table (or NULL; ft_decode_programs and ft_decode_static) holds one record of 16 int32 per
+ * request for the second launch: req_to_vnode_lens[r], req_to_vnode_offs[r], then the first 14
+ * entries of the request's part of req_to_vnode_entries (unused entries anything).  A block of the
+ * second launch then knows which partial rows to ask for after one memory round trip instead of two
+ * (length and offset, then the entries); entries beyond the fourteenth are read from the list.
+ * Trusted like the lists.
  */
 int ft_stage1_programs(const void* q, const void* k, const void* v,
                        int64_t sq0, int64_t sq1, int64_t sk0, int64_t sk1, int64_t sv0, int64_t sv1,
@@ -165,7 +172,7 @@ int ft_decode_programs(const void* q, const void* k, const void* v, void* o,
                        float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
                        const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
                        const int32_t* prog_table, int num_programs, int narrow_in_programs,
-                       const int32_t* narrow_table,
+                       const int32_t* narrow_table, const int32_t* req_table,
                        int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
                        float sm_scale, int dtype, ft_stream_t stream);
 
@@ -206,7 +213,7 @@ int ft_decode_static(const void* q, const void* k, const void* v, void* o,
                      const int32_t* req_to_vnode_lens, int64_t num_rows,
                      const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
                      const int32_t* prog_table, int num_programs, int narrow_in_programs,
-                     const int32_t* narrow_table,
+                     const int32_t* narrow_table, const int32_t* req_table,
                      int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
                      float sm_scale, int dtype, ft_stream_t stream);
 

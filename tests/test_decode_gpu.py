@@ -552,6 +552,31 @@ def test_narrow_vnode_wider_than_its_tile_argument_with_shared_waves(device):
 
 
 @pytest.mark.gpu
+def test_request_records_do_not_change_the_result(device):
+    """The merge launch with the per-request records (row count, offset and the first 14 scratch
+    rows in one place) gives bit for bit what it gives from the lists alone -- also for requests
+    with more rows than a record holds (a chain of 20 nodes: 20 rows and more per request)."""
+    _announce("request records")
+    scale = 1.0 / math.sqrt(128)
+    for sizes, lens, splits in (([1, 4, 40], [900, 100, 30], [256, 128]), ([1] * 19 + [6], [70] * 19 + [33], [1024, 256])):
+        tree, ptrs, batch = build_tree({"kind": "regular", "sizes": sizes, "lens": lens})
+        inp = make_decode_inputs(tree, 32, 8, 128, device=device, dtype=torch.float16, seed=11, shuffle_slots=True)
+        params = FastTreeParams()
+        params.set_values(0.66, 0.33, -10.0)      # (no node is merged into its children: a row per node)
+        params.set_q_tile_sizes([16, 4]); params.set_kv_tile_sizes([32, 32]); params.set_kv_group_num(4)
+        aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, 32, 8, 128, splits, [256, 1024], [256, 256], params,
+                                      device=device, kv_slot_map=inp.slot_map, launch_order=True)
+        nums = aux[11]
+        assert nums.req_table is not None and int(aux[8].max()) > (14 if len(sizes) > 3 else 2)
+        with_records = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, list(params.TSQs), [32, 32], scale)
+        table, nums.req_table = nums.req_table, None
+        without = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, list(params.TSQs), [32, 32], scale)
+        nums.req_table = table
+        assert torch.equal(with_records, without)
+        _dense_check(tree, inp, with_records, f"request records {sizes}")
+
+
+@pytest.mark.gpu
 def test_decode_replays_from_a_captured_graph(device):
     """The decode call allocates nothing and only enqueues launches on the stream it is given, so
     a caller can capture it: the graph is replayed several times, with eager work, new inputs

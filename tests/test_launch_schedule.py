@@ -310,3 +310,45 @@ def test_narrow_records_repeat_the_lists(monkeypatch):
             assert table[i, 4:4 + min(q_lens[v], 16)].tolist() == q_entries[q_offs[v]: q_offs[v] + min(q_lens[v], 16)].tolist()
             want = [kv_entries[kv_offs[v] + min(t, kv_lens[v] - 1)] for t in range(32)]
             assert table[i, 20:52].tolist() == want
+        # the per-request records of the merge launch: length, offset, the first 14 scratch rows
+        req_entries, req_offs, req_lens = (t.numpy() for t in aux[6:9])
+        records = nums.req_table.view(-1, 16).numpy()
+        assert records.shape[0] == batch
+        for r in range(0, batch, max(1, batch // 60)):
+            n, off = int(req_lens[r]), int(req_offs[r])
+            assert records[r, :2].tolist() == [n, off]
+            assert records[r, 2:2 + min(n, 14)].tolist() == req_entries[off: off + min(n, 14)].tolist()
+
+
+def test_request_records_by_hand():
+    rec = ls.request_records([5, 6, 7, 9, 1, 2, 3, -1, -1], [0, 3, 4], [3, 1, 3])
+    assert rec.shape == (3, 16) and rec.dtype == np.int32
+    assert rec[0].tolist() == [3, 0, 5, 6, 7] + [0] * 11
+    assert rec[1].tolist() == [1, 3, 9] + [0] * 13
+    assert rec[2].tolist() == [3, 4, 1, 2, 3] + [0] * 11
+    long = ls.request_records(list(range(100, 130)), [0, 20], [20, 10])      # more rows than a record holds
+    assert long[0].tolist() == [20, 0] + list(range(100, 114))
+    assert long[1].tolist() == [10, 20] + list(range(120, 130)) + [0] * 4
+    assert ls.request_records([], [], []).shape == (0, 16)
+    assert ls.request_records([], [0], [0])[0].tolist() == [0] * 16          # a request without rows
+
+
+def test_modelled_duration_of_narrow_launches_by_hand():
+    """The modelled duration of launches of narrow vnodes alone, worked by hand: ten vnodes of four
+    tiles leave the wave slots empty, so four waves share each (one tile step per wave, plus the
+    merge of the four); 2000 vnodes of one tile for one kv head fill the slots, one wave each; with
+    eight kv heads they take eight rounds' worth of the slots."""
+    us = ls.TILE_US_SHARED
+    few = ls.block_programs([128 * i for i in range(10)], [128] * 10, list(range(10)), [1] * 10, list(range(10)), 10, 16, 1,
+                            num_cus=256)
+    assert few.phase_node_nums == [0, 10]
+    want = (ls.NARROW_STARTUP_TILES + ls.NARROW_STEP_TILES * 1 + ls.NARROW_SHARE_TILES) * us + ls.LAUNCH_US
+    assert few.modelled_us == pytest.approx(want)
+    n = 2000
+    many = ls.block_programs([32 * i for i in range(n)], [32] * n, list(range(n)), [1] * n, list(range(n)), n, 16, 1, num_cus=256)
+    item = (ls.NARROW_STARTUP_TILES + ls.NARROW_STEP_TILES) * us
+    stream = n * 32 * 4 * 128 / ls.NARROW_BYTES_PER_US                       # K and V rows of one head at the narrow rate
+    assert item < stream < 1.1 * item
+    assert many.modelled_us == pytest.approx(stream + ls.LAUNCH_US)          # 2000 waves on 2048 slots: one item, or its bytes
+    eight = ls.block_programs([32 * i for i in range(n)], [32] * n, list(range(n)), [1] * n, list(range(n)), n, 4, 8, num_cus=256)
+    assert eight.modelled_us == pytest.approx(max(item * n * 8 / 2048, 8 * stream) + ls.LAUNCH_US)
