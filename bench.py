@@ -214,6 +214,7 @@ def main():
         if args.phase == "wide":
             part.prog_table = getattr(nums, "prog_table", None)
             part.num_programs = getattr(nums, "num_programs", 0)
+            part.prog_records = getattr(nums, "prog_records", None)
         elif getattr(nums, "narrow_in_programs", 0):
             log("bench.py: the narrow vnodes of this plan are served inside the block programs")
             sys.exit(2)

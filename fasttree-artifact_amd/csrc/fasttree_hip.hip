@@ -144,6 +144,9 @@ struct Stage1Args {
   // what a wave needs to start on the vnode in one memory round trip instead of two -- the vnode's
   // four list entries, the requests of its rows and the pool slots of its first 32 tokens
   const int32_t* narrow_table;
+  // one record of kProgRecord ints per program, written by the host (or null): what the block needs to
+  // start on the program's first wide vnode -- see kProgRecord
+  const int32_t* prog_records;
   int real_dim;                    // head dimension of the tensors; smaller than the kernel's D only for head_dim 16,
                                    // which the per-wave staging kernels compute as a zero-padded 32-dim contraction
   int g;
@@ -542,7 +545,8 @@ template <int D> struct WideGeom {
   static constexpr int kUnits = 2 * kGroups / kWideWaves;                       // loads per wave and super tile
   static constexpr int kSlots = kGroups >= kWideWaves ? kGroups / kWideWaves : 1;  // distinct rows among them
   static constexpr int kIdxCap = 2048;                    // slot indices staged at a time (tokens)
-  static constexpr int kLds = kRing + 4 * kIdxCap;
+  static constexpr int kRecord = kRing + 4 * kIdxCap;    // byte offset of the program's record (kProgRecord ints)
+  static constexpr int kLds = kRecord + 1024;
   static __device__ __forceinline__ int swz(int row) { return (((row & 3) << 2) | ((row >> 2) & 3)) & (kChunks - 1); }
 };
 
@@ -569,14 +573,29 @@ __device__ __forceinline__ void reset_state(WideState<D>& st) {
 // between the two dependent ones: the address of a lane's row (needs the request id of the row,
 // one load), then the fragments.  qf[ks]: row row0 + lane%32, dims 16*ks + 8*(lane/32) .. +7;
 // zero past the vnode (src == nullptr).
+// The record of a block program (kProgRecord ints, one thread of the block each): entries 0..3 are
+// kv_off, kv_len, q_off and q_len of the program's first wide vnode, entry 4 says whether the rest is
+// there (the vnode exists and has at most kWideRows query rows), entries kProgRecRequests.. the
+// requests of its scratch rows, entries kProgRecSlots.. the pool slots of its first 64 tokens (the
+// last token repeated past the end of a shorter run).  With it a block knows after one memory round
+// trip what it otherwise learns in three (its table entry, the vnode's list entries, the request
+// and slot lists) before it can ask for query and K/V rows.
+constexpr int kProgRecord = 256;
+constexpr int kProgRecRequests = 8;
+constexpr int kProgRecSlots = kProgRecRequests + 128;
+static_assert(kProgRecSlots + 64 <= kProgRecord && kProgRecord == 4 * 64, "one entry per thread of a block");
+
+// (requests: the record's request entries in LDS, or null: the request of a row is read from the list)
 template <bool GATHERED>
-__device__ __forceinline__ const char* q_row_address32(const Stage1Args& a, const VnodeView& vn, int kvh, int row0) {
+__device__ __forceinline__ const char* q_row_address32(const Stage1Args& a, const VnodeView& vn, int kvh, int row0,
+                                                       const int* requests = nullptr) {
   const int lane = threadIdx.x & 63;
   const int r = row0 + (lane & 31), h = lane >> 5;
   if (r >= vn.q_len * a.g) return nullptr;
   const int ri = r / a.g;
   const int rj = r - ri * a.g;
-  const int64_t entry = GATHERED ? (int64_t)(vn.q_off / a.nsplit) : (int64_t)a.q_entries[vn.q_off + ri];
+  const int64_t entry = GATHERED ? (int64_t)(vn.q_off / a.nsplit)
+                                 : (int64_t)(requests ? requests[ri] : a.q_entries[vn.q_off + ri]);
   return a.q + 2 * (entry * a.sq0 + (int64_t)(kvh * a.g + rj) * a.sq1 + 8 * h);
 }
 template <int D>
@@ -830,7 +849,7 @@ __device__ __forceinline__ void merge_token_groups(float* xchg, WideState<D>& st
 // its row group, and the TG states of a row group are merged at the end.
 template <typename E, int D, bool GATHERED>
 __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, const VnodeView& vn, int kvh, int chunk,
-                                           int chunks) {
+                                           int chunks, const int* record = nullptr) {
   using W = WideGeom<D>;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int rows_total = vn.q_len * a.g;
@@ -861,7 +880,11 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, cons
     const bool active = rg < rgroups && my_row0 < rows_end;
 
     // start-up chain: [request ids of the rows, slot indices] -> [Q fragments, first K/V rows]
-    const char* q_src = q_row_address32<GATHERED>(a, vn, kvh, active ? my_row0 : rows_total);
+    // (the program's record covers the vnode's first kWideRows rows: its first piece, one pass)
+    // (not at head_dim 256, where the step has no register to spare)
+    const int* rec = (!GATHERED && D <= 128 && piece == 0) ? record : nullptr;   // block uniform
+    const char* q_src = q_row_address32<GATHERED>(a, vn, kvh, active ? my_row0 : rows_total,
+                                                  rec ? rec + kProgRecRequests : nullptr);
     u32x4 qf[D / 16];
     WideState<D> st;
     reset_state<D>(st);
@@ -919,11 +942,24 @@ __device__ __forceinline__ void wide_block(const Stage1Args& a, char* smem, cons
         load_direct16(src + 16 * (pos ^ W::swz(row)), buf + (is_v ? W::kBytesK : 0) + grp * 1024);
       }
     };
-    if (nsuper > 0) stage_indices(0);  // block uniform
+    static_assert(W::kAhead == 1, "the record path below requests exactly the first super tile");
+    if (rec && nsuper > 0) {
+      // the first super tile's slots come with the record: its rows are requested before the
+      // run's index list has been read at all
 #pragma unroll
-    for (int j = 0; j < W::kAhead; ++j) {
-      read_rows(j);
-      issue_rows(j);
+      for (int u = 0; u < W::kSlots; ++u) {
+        const int grp = W::kGroups >= kWideWaves ? u * kWideWaves + wave : wave % W::kGroups;
+        srow[u] = (unsigned)rec[kProgRecSlots + grp * W::kGroupRows + grp_row];
+      }
+      issue_rows(0);
+      stage_indices(0);
+    } else {
+      if (nsuper > 0) stage_indices(0);  // block uniform
+#pragma unroll
+      for (int j = 0; j < W::kAhead; ++j) {
+        read_rows(j);
+        issue_rows(j);
+      }
     }
     read_rows(W::kAhead);
     load_q_frags32<D>(q_src, qf);
@@ -1414,10 +1450,22 @@ __global__ void __launch_bounds__(kWideBlock, D > 128 ? 1 : 512 / kWideBlock) st
         narrow_item<E, D, GATHERED>(a, smem, wave, 1, true, a.narrow_begin + narrow_first + i, kvh);
       __syncthreads();  // the waves' tiles become the ring of the next wide vnode
     };
+    // the program's record, requested together with its table entry
+    int* record = reinterpret_cast<int*>(smem + WideGeom<D>::kRecord);
+    const bool with_records = !GATHERED && D <= 128 && a.prog_records != nullptr;   // launch uniform
+    if (with_records) {
+      record[threadIdx.x] = a.prog_records[(int64_t)program * kProgRecord + threadIdx.x];
+      __syncthreads();
+    }
     if (narrow_signed < 0) narrow_vnodes();
     for (int v = wide_first; v < wide_end; ++v) {
-      const VnodeView vn = load_vnode<GATHERED>(a, a.vnode_begin + v);
-      wide_block<E, D, GATHERED>(a, smem, vn, kvh, 0, 1);
+      if (with_records && narrow_signed >= 0 && v == wide_first && record[4] != 0) {
+        const VnodeView vn{record[2], record[3], record[1], (int64_t)record[0]};
+        wide_block<E, D, GATHERED>(a, smem, vn, kvh, 0, 1, record);
+      } else {
+        const VnodeView vn = load_vnode<GATHERED>(a, a.vnode_begin + v);
+        wide_block<E, D, GATHERED>(a, smem, vn, kvh, 0, 1);
+      }
     }
     if (narrow_signed > 0) narrow_vnodes();
   } else if (is_wide) {
@@ -2139,7 +2187,7 @@ int ft_stage1_programs(const void* q, const void* k, const void* v,
                        float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
                        const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
                        const int32_t* prog_table, int num_programs, int narrow_in_programs,
-                       const int32_t* narrow_table,
+                       const int32_t* narrow_table, const int32_t* prog_records,
                        int num_qo_heads, int num_kv_heads, int head_dim,
                        float sm_scale, int dtype, ft_stream_t stream) {
   if (!phase_node_nums || !phase_node_offsets) return FT_ERR_NULL_POINTER;
@@ -2163,6 +2211,7 @@ int ft_stage1_programs(const void* q, const void* k, const void* v,
   a.narrow_begin = phase_node_offsets[1]; a.narrow_count = phase_node_nums[1];
   if (num_programs > 0) { a.prog_table = prog_table; a.num_programs = num_programs; a.narrow_in_programs = narrow_in_programs; }
   a.narrow_table = narrow_table;
+  a.prog_records = num_programs > 0 ? prog_records : nullptr;
   a.wide_rows = kWideRows;
   return launch_stage1<false>(a, head_dim, dtype, stream);
 }
@@ -2178,14 +2227,14 @@ int ft_decode_programs(const void* q, const void* k, const void* v, void* o,
                        float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
                        const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
                        const int32_t* prog_table, int num_programs, int narrow_in_programs,
-                       const int32_t* narrow_table, const int32_t* req_table,
+                       const int32_t* narrow_table, const int32_t* prog_records, const int32_t* req_table,
                        int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
                        float sm_scale, int dtype, ft_stream_t stream) {
   if (int rc = ft_stage1_programs(q, k, v, sq0, sq1, sk0, sk1, sv0, sv1, vnode_to_kv_entries, vnode_to_kv_offs,
                                   vnode_to_kv_lens, vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, mid_o, so0,
                                   so1, mid_lse, sl0, phase_node_nums, phase_node_offsets, prog_table, num_programs,
-                                  narrow_in_programs, narrow_table, num_qo_heads, num_kv_heads, head_dim, sm_scale, dtype,
-                                  stream))
+                                  narrow_in_programs, narrow_table, prog_records, num_qo_heads, num_kv_heads, head_dim,
+                                  sm_scale, dtype, stream))
     return rc;
   return stage2_with_table(req_to_vnode_entries, req_to_vnode_offs, req_to_vnode_lens, req_table, mid_o, so0, so1,
                            mid_lse, sl0, o, oo0, oo1, batch_size, num_qo_heads, head_dim, dtype, stream);
@@ -2201,7 +2250,7 @@ int ft_decode_static(const void* q, const void* k, const void* v, void* o,
                      const int32_t* req_to_vnode_lens, int64_t num_rows,
                      const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
                      const int32_t* prog_table, int num_programs, int narrow_in_programs,
-                     const int32_t* narrow_table, const int32_t* req_table,
+                     const int32_t* narrow_table, const int32_t* prog_records, const int32_t* req_table,
                      int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
                      float sm_scale, int dtype, ft_stream_t stream) {
   if (num_rows < 0 || num_qo_heads < 1 || head_dim < 1) return FT_ERR_ARGUMENT;
@@ -2218,7 +2267,7 @@ int ft_decode_static(const void* q, const void* k, const void* v, void* o,
                             vnode_to_kv_lens, vnode_to_q_entries, vnode_to_q_offs, vnode_to_q_lens, req_to_vnode_entries,
                             req_to_vnode_offs, req_to_vnode_lens, mid_o, (int64_t)num_qo_heads * head_dim, head_dim,
                             mid_lse, num_qo_heads, phase_node_nums, phase_node_offsets, prog_table, num_programs,
-                            narrow_in_programs, narrow_table, req_table, batch_size, num_qo_heads, num_kv_heads, head_dim,
+                            narrow_in_programs, narrow_table, prog_records, req_table, batch_size, num_qo_heads, num_kv_heads, head_dim,
                             sm_scale, dtype, stream);
 }
 

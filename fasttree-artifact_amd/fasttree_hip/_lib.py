@@ -34,12 +34,12 @@ SIGNATURES = {
     "ft_decode": (c_int, [_P, _P, _P, _P] + [c_int64] * 8 + [_P] * 9
                   + [_P, c_int64, c_int64, _P, c_int64] + [_P] * 4 + [c_int] * 4 + [c_float, c_int, _P]),
     "ft_stage1_programs": (c_int, [_P, _P, _P] + _I64x6 + [_P] * 6 + [_P, c_int64, c_int64, _P, c_int64] + [_P] * 2
-                           + [_P, c_int, c_int, _P] + [c_int] * 3 + [c_float, c_int, _P]),
+                           + [_P, c_int, c_int, _P, _P] + [c_int] * 3 + [c_float, c_int, _P]),
     "ft_decode_programs": (c_int, [_P, _P, _P, _P] + [c_int64] * 8 + [_P] * 9
-                           + [_P, c_int64, c_int64, _P, c_int64] + [_P] * 2 + [_P, c_int, c_int, _P, _P] + [c_int] * 4
+                           + [_P, c_int64, c_int64, _P, c_int64] + [_P] * 2 + [_P, c_int, c_int, _P, _P, _P] + [c_int] * 4
                            + [c_float, c_int, _P]),
     "ft_decode_static": (c_int, [_P, _P, _P, _P] + [c_int64] * 8 + [_P] * 9 + [c_int64] + [_P] * 2
-                         + [_P, c_int, c_int, _P, _P] + [c_int] * 4 + [c_float, c_int, _P]),
+                         + [_P, c_int, c_int, _P, _P, _P] + [c_int] * 4 + [c_float, c_int, _P]),
     "ft_deft_stage1": (c_int, [_P, _P, _P] + _I64x6 + [_P] * 6 + [_P, _P] + [c_int] * 5 + [c_float]
                        + [_P, c_int64, c_int64, _P, c_int64, c_int, _P]),
     "ft_deft_decode": (c_int, [_P, _P, _P, _P] + [c_int64] * 8 + [_P] * 6 + [_P, _P] + [_P] * 3

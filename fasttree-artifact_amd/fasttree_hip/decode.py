@@ -32,6 +32,12 @@ def _narrow_table_ptr(phase_node_nums):
     return table.data_ptr() if table is not None else None
 
 
+def _prog_records_ptr(phase_node_nums):
+    """Device pointer of the records of the block programs a launch-order plan carries, or None."""
+    table = getattr(phase_node_nums, "prog_records", None)
+    return table.data_ptr() if table is not None and getattr(phase_node_nums, "prog_table", None) is not None else None
+
+
 def _req_table_ptr(phase_node_nums):
     """Device pointer of the per-request records for the merge launch, or None."""
     table = getattr(phase_node_nums, "req_table", None)
@@ -95,7 +101,7 @@ def fasttree_decode(
             programs.data_ptr() if programs is not None else None,
             int(phase_node_nums.num_programs) if programs is not None else 0,
             int(phase_node_nums.narrow_in_programs) if programs is not None else 0, narrow_table,
-            _req_table_ptr(phase_node_nums),
+            _prog_records_ptr(phase_node_nums), _req_table_ptr(phase_node_nums),
             q.shape[0], q.shape[1], k_buffer.shape[1], q.shape[-1],
             float(sm_scale), _dtype_code(q), _stream_handle(q),
         )
@@ -150,7 +156,7 @@ def fasttree_decode_static(q, k_buffer, v_buffer, o, vnode_to_kv_entries, vnode_
         programs.data_ptr() if programs is not None else None,
         int(getattr(phase_node_nums, "num_programs", 0)) if programs is not None else 0,
         int(getattr(phase_node_nums, "narrow_in_programs", 0)) if programs is not None else 0,
-        _narrow_table_ptr(phase_node_nums), _req_table_ptr(phase_node_nums),
+        _narrow_table_ptr(phase_node_nums), _prog_records_ptr(phase_node_nums), _req_table_ptr(phase_node_nums),
         q.shape[0], q.shape[1], k_buffer.shape[1], q.shape[-1],
         float(sm_scale), _dtype_code(q), _stream_handle(q),
     )
@@ -177,6 +183,7 @@ def fasttree_decode_stage1(q, k_buffer, v_buffer, vnode_to_kv_entries, vnode_to_
             programs.data_ptr() if programs is not None else None,
             int(phase_node_nums.num_programs) if programs is not None else 0,
             int(phase_node_nums.narrow_in_programs) if programs is not None else 0, narrow_table,
+            _prog_records_ptr(phase_node_nums),
             q.shape[1], k_buffer.shape[1], q.shape[-1], float(sm_scale), _dtype_code(q), _stream_handle(q),
         )
         _lib.check(rc, "ft_stage1_programs")

@@ -149,6 +149,8 @@ class LaunchPhases(list):
     narrow_table = None
     #: int32 device tensor of :func:`request_records` (16 entries per request), or None
     req_table = None
+    #: int32 device tensor of :func:`program_records` (256 entries per program), or None
+    prog_records = None
     #: what the schedule's model expects the first-stage launch to take, and the machine it was laid out for
     modelled_us = None
     num_cus = None
@@ -187,6 +189,8 @@ class LaunchSchedule:
 USE_NARROW_RECORDS = True
 #: Whether they carry the records of :func:`request_records` for the merge launch (likewise).
 USE_REQUEST_RECORDS = True
+#: Whether they carry the records of :func:`program_records` (likewise).
+USE_PROGRAM_RECORDS = True
 #: Entries of a narrow vnode's record, requests and token slots it holds (the kernels' layout).
 NARROW_RECORD = 64
 NARROW_RECORD_REQUESTS = 16
@@ -216,6 +220,48 @@ def narrow_records(kv_entries, kv_offs, kv_lens, q_offs, q_lens, q_entries, firs
     first_slot = 4 + NARROW_RECORD_REQUESTS
     table[:, first_slot:first_slot + NARROW_RECORD_TOKENS] = np.where(
         kl[:, None] > 0, kv_entries[np.minimum(tokens, max(len(kv_entries) - 1, 0))], 0) if len(kv_entries) else 0
+    return table
+
+
+#: Entries of a block program's record, where the requests and the token slots start in it, and how
+#: many rows and tokens they cover (the kernels' layout).
+PROGRAM_RECORD = 256
+PROGRAM_RECORD_REQUESTS = 8
+PROGRAM_RECORD_SLOTS = 136
+PROGRAM_RECORD_ROWS = 128
+PROGRAM_RECORD_TOKENS = 64
+
+
+def program_records(kv_entries, kv_offs, kv_lens, q_offs, q_lens, q_entries, prog_table, first, group):
+    """One record per block program: what its block needs to start on the program's first wide
+    vnode, in one place, so that it can ask for query and K/V rows after one memory round trip
+    (the record, fetched together with the table entry) instead of three (table entry, the
+    vnode's list entries, its request and slot lists).  Entries: ``kv_off, kv_len, q_off, q_len`` of
+    vnode ``first + prog_table[p][0]``; a flag (1: the program has a wide vnode of at most 128 query
+    rows and the rest is filled in); from entry 8 the requests of its scratch rows; from entry 136
+    the pool slots of its first 64 tokens (the last token repeated past the end of a shorter run).
+    Returns an int32 array ``[num_programs, 256]``."""
+    prog_table = np.asarray(prog_table, dtype=np.int64).reshape(-1, 4)
+    kv_entries = np.asarray(kv_entries).reshape(-1)
+    q_entries = np.asarray(q_entries).reshape(-1)
+    table = np.zeros((len(prog_table), PROGRAM_RECORD), dtype=np.int32)
+    if len(prog_table) == 0:
+        return table
+    has = prog_table[:, 1] > prog_table[:, 0]
+    v = np.where(has, int(first) + prog_table[:, 0], 0)
+    take = lambda x: np.asarray(x, dtype=np.int64).reshape(-1)[v] if len(x) else np.zeros(len(v), dtype=np.int64)
+    ko, kl, qo, ql = take(kv_offs), take(kv_lens), take(q_offs), take(q_lens)
+    ok = has & (ql * int(group) <= PROGRAM_RECORD_ROWS) & (ql > 0)
+    table[:, 0], table[:, 1], table[:, 2], table[:, 3], table[:, 4] = ko, kl, qo, ql, ok
+    if len(q_entries):
+        rows = qo[:, None] + np.minimum(np.arange(PROGRAM_RECORD_ROWS)[None, :], np.maximum(ql[:, None] - 1, 0))
+        table[:, PROGRAM_RECORD_REQUESTS:PROGRAM_RECORD_REQUESTS + PROGRAM_RECORD_ROWS] = np.where(
+            ok[:, None], q_entries[np.minimum(rows, len(q_entries) - 1)], 0)
+    if len(kv_entries):
+        tokens = ko[:, None] + np.minimum(np.arange(PROGRAM_RECORD_TOKENS)[None, :], np.maximum(kl[:, None] - 1, 0))
+        table[:, PROGRAM_RECORD_SLOTS:PROGRAM_RECORD_SLOTS + PROGRAM_RECORD_TOKENS] = np.where(
+            (ok & (kl > 0))[:, None], kv_entries[np.minimum(tokens, len(kv_entries) - 1)], 0)
+    table[~ok, 4] = 0
     return table
 
 

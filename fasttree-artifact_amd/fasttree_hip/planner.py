@@ -449,6 +449,7 @@ class PlanBuffers:
         self.prog_table = ints(4 * max_vnodes)
         self.narrow_table = ints(64 * max_vnodes)     # (launch_schedule.NARROW_RECORD entries per narrow vnode)
         self.req_table = ints(16 * max_batch_size)    # (launch_schedule.REQUEST_RECORD entries per request)
+        self.prog_records = ints(256 * max_vnodes)    # (launch_schedule.PROGRAM_RECORD entries per program)
         self.mid_o = torch.empty((int(max_rows), num_qo_heads, head_dim), dtype=torch.float32, device=device)
         self.mid_lse = torch.empty((int(max_rows), num_qo_heads), dtype=torch.float32, device=device)
 
@@ -544,6 +545,10 @@ def fasttree_preparation(
             phase_nums.num_programs = sched.num_programs
             phase_nums.narrow_in_programs = sched.narrow_in_programs
         from . import launch_schedule
+        if sched.num_programs > 0 and head_dim >= 32 and launch_schedule.USE_PROGRAM_RECORDS:
+            records = launch_schedule.program_records(plan.vnode_to_kv_entries, *vnodes, q_entries, sched.prog_table,
+                                                      phase_offs[0], group)
+            phase_nums.prog_records = place("prog_records", records.reshape(-1))
         if phase_nums[1] > 0 and head_dim >= 32 and launch_schedule.USE_NARROW_RECORDS:
             from .launch_schedule import narrow_records
             records = narrow_records(plan.vnode_to_kv_entries, *vnodes, q_entries, phase_offs[1], phase_nums[1])

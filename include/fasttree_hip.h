@@ -142,6 +142,15 @@ int ft_decode(const void* q, const void* k, const void* v, void* o,
  * list entries, then the index and request lists) before it can ask for K/V rows.  The records must
  * agree with the lists; they are trusted like them.
  *
+ * prog_records (or NULL) holds one record of 256 int32 per program: entries 0..3 the kv_off, kv_len,
+ * q_off and q_len of the program's first vnode of the first range; entry 4 is 1 when the rest is filled
+ * in (the program has such a vnode and it has at most 128 query rows = q_len * group), else 0; entries
+ * 8..135 the requests of its scratch rows (vnode_to_q_entries[q_off ...]); entries 136..199 the pool slots
+ * of its first 64 tokens (vnode_to_kv_entries[kv_off + min(t, kv_len - 1)]); the rest is padding.  A block
+ * then asks for the query and K/V rows of its first vnode after one memory round trip (record and table
+ * entry together) instead of three (table entry, list entries, request and slot lists).  Trusted like the
+ * lists.
+ *
  * req_table (or NULL; ft_decode_programs and ft_decode_static) holds one record of 16 int32 per
  * request for the second launch: req_to_vnode_lens[r], req_to_vnode_offs[r], then the first 14
  * entries of the request's part of req_to_vnode_entries (unused entries anything).  A block of the
@@ -157,7 +166,7 @@ int ft_stage1_programs(const void* q, const void* k, const void* v,
                        float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
                        const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
                        const int32_t* prog_table, int num_programs, int narrow_in_programs,
-                       const int32_t* narrow_table,
+                       const int32_t* narrow_table, const int32_t* prog_records,
                        int num_qo_heads, int num_kv_heads, int head_dim,
                        float sm_scale, int dtype, ft_stream_t stream);
 
@@ -172,7 +181,7 @@ int ft_decode_programs(const void* q, const void* k, const void* v, void* o,
                        float* mid_o, int64_t so0, int64_t so1, float* mid_lse, int64_t sl0,
                        const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
                        const int32_t* prog_table, int num_programs, int narrow_in_programs,
-                       const int32_t* narrow_table, const int32_t* req_table,
+                       const int32_t* narrow_table, const int32_t* prog_records, const int32_t* req_table,
                        int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
                        float sm_scale, int dtype, ft_stream_t stream);
 
@@ -213,7 +222,7 @@ int ft_decode_static(const void* q, const void* k, const void* v, void* o,
                      const int32_t* req_to_vnode_lens, int64_t num_rows,
                      const int32_t phase_node_nums[2], const int32_t phase_node_offsets[2],
                      const int32_t* prog_table, int num_programs, int narrow_in_programs,
-                     const int32_t* narrow_table, const int32_t* req_table,
+                     const int32_t* narrow_table, const int32_t* prog_records, const int32_t* req_table,
                      int batch_size, int num_qo_heads, int num_kv_heads, int head_dim,
                      float sm_scale, int dtype, ft_stream_t stream);
 

@@ -577,6 +577,38 @@ def test_request_records_do_not_change_the_result(device):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("d,dtype", [(128, torch.float16), (64, torch.bfloat16), (256, torch.float16), (32, torch.float16)])
+def test_program_records_do_not_change_the_result(d, dtype, device):
+    """Block programs that start from their record (list entries, requests and the first 64 slots of
+    the first wide vnode in one place) give bit for bit what they give from the lists alone: runs
+    shorter than a super tile, of exactly 64 tokens, with a last tile of one token, a vnode of more
+    than 128 rows (no record), programs of several vnodes."""
+    _announce("program records", d, dtype)
+    scale = 1.0 / math.sqrt(d)
+    for sizes, lens, heads in (([1, 4, 40], [900, 100, 30], (32, 8)), ([1, 3, 60], [33, 64, 5], (32, 8)),
+                               ([1, 2, 70], [257, 40, 12], (16, 16)), ([1, 8, 48, 96], [2100, 130, 65, 20], (32, 4))):
+        tree, ptrs, batch = build_tree({"kind": "regular", "sizes": sizes, "lens": lens})
+        hq, hkv = heads
+        g = hq // hkv
+        inp = make_decode_inputs(tree, hq, hkv, d, device=device, dtype=dtype, seed=5, shuffle_slots=True)
+        params = FastTreeParams()
+        params.set_values(0.66, 0.33, 0.1)
+        params.set_q_tile_sizes([max(1, 64 // g), max(1, 16 // g)]); params.set_kv_tile_sizes([32, 32]); params.set_kv_group_num(g)
+        aux, _ = fasttree_preparation(tree, inp.KV_ptrs, batch, hq, hkv, d, [1024, 256], [256, 1024], [256, 256], params,
+                                      device=device, kv_slot_map=inp.slot_map, launch_order=True)
+        nums = aux[11]
+        if getattr(nums, "prog_table", None) is None:
+            continue
+        assert nums.prog_records is not None
+        with_records = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, list(params.TSQs), [32, 32], scale)
+        records, nums.prog_records = nums.prog_records, None
+        without = _decode(inp.Q, inp.K_pool, inp.V_pool, aux, list(params.TSQs), [32, 32], scale)
+        nums.prog_records = records
+        assert torch.equal(with_records, without), f"{sizes} {heads}"
+        _dense_check(tree, inp, with_records, f"program records {sizes} {heads} d{d}", dtype=dtype, aux=aux)
+
+
+@pytest.mark.gpu
 def test_decode_replays_from_a_captured_graph(device):
     """The decode call allocates nothing and only enqueues launches on the stream it is given, so
     a caller can capture it: the graph is replayed several times, with eager work, new inputs

@@ -320,6 +320,51 @@ def test_narrow_records_repeat_the_lists(monkeypatch):
             assert records[r, 2:2 + min(n, 14)].tolist() == req_entries[off: off + min(n, 14)].tolist()
 
 
+def test_program_records_repeat_the_lists(monkeypatch):
+    """The record of a block program holds what the lists say about its first wide vnode: the four
+    list entries, the requests of its rows, the pool slots of its first 64 tokens (the last one
+    repeated past a shorter run); programs without a wide vnode, or with one of more than 128 query
+    rows, are flagged as having none (hand case, then the programs of three launch-order plans)."""
+    kv_entries = np.arange(500, 800)
+    #             vnode:   0    1    2
+    kv_offs, kv_lens = [0, 100, 130], [100, 30, 70]
+    q_offs, q_lens = [0, 40, 43], [40, 3, 33]
+    q_entries = list(range(900, 976))
+    table = [[1, 2, 0, 0], [0, 1, 0, 0], [2, 2, 0, 0], [2, 3, 0, 0]]       # programs: vnode 1; vnode 0; none; vnode 2
+    rec = ls.program_records(kv_entries, kv_offs, kv_lens, q_offs, q_lens, q_entries, table, 0, 4)
+    assert rec.shape == (4, 256) and rec.dtype == np.int32
+    assert rec[0, :5].tolist() == [100, 30, 40, 3, 1]
+    assert rec[0, 8:11].tolist() == [940, 941, 942]
+    assert rec[0, 136:200].tolist() == list(range(600, 630)) + [629] * 34
+    assert rec[1, :5].tolist() == [0, 100, 0, 40, 0]                       # 40 requests x 4 heads: more than 128 rows
+    assert rec[2, 4] == 0 and rec[3, :5].tolist() == [130, 70, 43, 33, 0]  # no wide vnode; 132 rows
+    assert ls.program_records(kv_entries, kv_offs, kv_lens, q_offs, q_lens, q_entries, table, 0, 1)[1, 4] == 1
+    assert ls.program_records([], [], [], [], [], [], np.zeros((0, 4)), 0, 4).shape == (0, 256)
+    import fasttree_hip.planner as planner_module
+    from fasttree_hip.planner import FastTreeParams, fasttree_preparation
+    monkeypatch.setattr(planner_module, "VERBOSE", False)
+    for name in ("c3", "c5_seed0", "c2"):
+        case = next(c for c in PLANNER_CASES if c["name"] == name)
+        tree, ptrs, batch = build_tree(case["tree"])
+        g = case["Hq"] // case["Hkv"]
+        p = FastTreeParams(); p.set_values(0.66, 0.33, 0.1); p.set_q_tile_sizes([max(1, 64 // g), max(1, 16 // g)])
+        p.set_kv_tile_sizes([32, 32]); p.set_kv_group_num(g)
+        slot_map = np.random.default_rng(0).permutation(ptrs[-1])
+        aux, _ = fasttree_preparation(tree, ptrs, batch, case["Hq"], case["Hkv"], 128, [1024, 256], [256, 1024], [256, 256], p,
+                                      device="cpu", kv_slot_map=slot_map, launch_order=True)
+        nums, offs = aux[11], aux[12]
+        records = nums.prog_records.view(-1, 256).numpy()
+        programs = nums.prog_table.view(-1, 4).numpy()
+        assert records.shape[0] == nums.num_programs == len(programs) > 0
+        kv_entries, kv_offs, kv_lens, q_entries, q_offs, q_lens = (t.numpy() for t in aux[:6])
+        assert records[:, 4].all()            # every program of these plans starts with a vnode of at most 128 rows
+        for i in range(0, len(programs), max(1, len(programs) // 40)):
+            v = offs[0] + programs[i, 0]
+            assert records[i, :4].tolist() == [kv_offs[v], kv_lens[v], q_offs[v], q_lens[v]]
+            assert records[i, 8:8 + q_lens[v]].tolist() == q_entries[q_offs[v]: q_offs[v] + q_lens[v]].tolist()
+            assert records[i, 136:200].tolist() == [kv_entries[kv_offs[v] + min(t, kv_lens[v] - 1)] for t in range(64)]
+
+
 def test_request_records_by_hand():
     rec = ls.request_records([5, 6, 7, 9, 1, 2, 3, -1, -1], [0, 3, 4], [3, 1, 3])
     assert rec.shape == (3, 16) and rec.dtype == np.int32

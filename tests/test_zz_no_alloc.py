@@ -74,7 +74,7 @@ def test_static_scratch_refuses_what_does_not_fit(device):
             inp.Q.stride(0), inp.Q.stride(1), inp.K_pool.stride(0), inp.K_pool.stride(1),
             inp.V_pool.stride(0), inp.V_pool.stride(1), o.stride(0), o.stride(1)]
     args += [t.data_ptr() for t in aux[:9]]
-    tail = [_lib.int32_pair(aux[11]), _lib.int32_pair(aux[12]), None, 0, 0, None, None, inp.Q.shape[0], 32, 8, 128,
+    tail = [_lib.int32_pair(aux[11]), _lib.int32_pair(aux[12]), None, 0, 0, None, None, None, inp.Q.shape[0], 32, 8, 128,
             1.0 / math.sqrt(128), 0, None]
     rc = lib.ft_decode_static(*args, rows, *tail)
     assert rc == -8 and b"static scratch" in lib.ft_error_string(rc)
