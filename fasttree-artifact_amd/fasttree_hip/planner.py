@@ -466,6 +466,87 @@ class PlanBuffers:
         return part
 
 
+def place_plan(kv_entries, vnodes, q_entries, per_request, phase_nums, phase_offs,
+               batch_size, num_qo_heads, num_kv_heads, head_dim, *,
+               device="cuda", launch_order=False, buffers=None, num_cus=None):
+    """The 13 arguments ``fasttree_decode`` takes after the output tensor, from vnode lists on the
+    host: ``kv_entries`` (flat pool slots), ``vnodes = (kv_offs, kv_lens, q_offs, q_lens)``,
+    ``q_entries`` (request of every scratch row), ``per_request = (entries, offs, lens)`` (scratch
+    rows of every request; ignored with ``launch_order``, which derives its own), the two phase
+    lists.  Places the nine int32 arrays and the two fp32 partial-result buffers on ``device`` (into
+    ``buffers`` if given).  With ``launch_order`` the lists are first arranged as block programs
+    (:func:`launch_schedule.block_programs`) for ``num_cus`` compute units, and ``phase_node_nums``
+    comes back as a list that also carries the program table and the host-written records."""
+    import torch
+
+    from .launch_schedule import LaunchPhases, block_programs
+
+    names = iter(("vnode_to_kv_entries", "vnode_to_kv_offs", "vnode_to_kv_lens", "vnode_to_q_entries", "vnode_to_q_offs",
+                  "vnode_to_q_lens", "req_to_vnode_entries", "req_to_vnode_offs", "req_to_vnode_lens"))
+
+    def place(name, values):
+        if buffers is not None:
+            return buffers.fill(name, values)
+        host = torch.from_numpy(np.ascontiguousarray(np.asarray(values, dtype=np.int32)))
+        return host.to(device)
+
+    def put(values):
+        return place(next(names), values)  # (the nine arrays are placed in this order below)
+
+    rows = int(len(np.asarray(q_entries).reshape(-1)))
+    if launch_order:
+        group = max(1, num_qo_heads // num_kv_heads)
+        if num_cus is None:
+            from .launch_schedule import compute_units
+            num_cus = compute_units(device)
+        sched = block_programs(*vnodes, q_entries, batch_size, group, num_kv_heads, head_dim=head_dim, num_cus=num_cus)
+        vnodes = (sched.kv_offs, sched.kv_lens, sched.q_offs, sched.q_lens)
+        q_entries = sched.q_entries
+        per_request = (sched.req_entries, sched.req_offs, sched.req_lens)
+        rows = sched.num_rows
+        phase_nums, phase_offs = LaunchPhases(sched.phase_node_nums), list(sched.phase_node_offsets)
+        phase_nums.modelled_us, phase_nums.num_cus, phase_nums.block_slots = sched.modelled_us, sched.num_cus, sched.block_slots
+        if sched.num_programs > 0:
+            phase_nums.prog_table = place("prog_table", sched.prog_table.reshape(-1))
+            phase_nums.num_programs = sched.num_programs
+            phase_nums.narrow_in_programs = sched.narrow_in_programs
+        from . import launch_schedule
+        if sched.num_programs > 0 and head_dim >= 32 and launch_schedule.USE_PROGRAM_RECORDS:
+            records = launch_schedule.program_records(kv_entries, *vnodes, q_entries, sched.prog_table,
+                                                      phase_offs[0], group)
+            phase_nums.prog_records = place("prog_records", records.reshape(-1))
+        if phase_nums[1] > 0 and head_dim >= 32 and launch_schedule.USE_NARROW_RECORDS:
+            from .launch_schedule import narrow_records
+            records = narrow_records(kv_entries, *vnodes, q_entries, phase_offs[1], phase_nums[1])
+            phase_nums.narrow_table = place("narrow_table", records.reshape(-1))
+        if head_dim >= 32 and launch_schedule.USE_REQUEST_RECORDS:
+            from .launch_schedule import request_records
+            phase_nums.req_table = place("req_table", request_records(*per_request).reshape(-1))
+    if buffers is not None:
+        if rows > buffers.mid_o.shape[0] or buffers.mid_o.shape[1:] != (num_qo_heads, head_dim):
+            raise ValueError(f"the scratch of the buffers ({tuple(buffers.mid_o.shape)}) does not hold "
+                             f"{rows} rows of {num_qo_heads} x {head_dim}")
+        mid_o, mid_lse = buffers.mid_o[:rows], buffers.mid_lse[:rows]
+    else:
+        mid_o = torch.empty((rows, num_qo_heads, head_dim), dtype=torch.float32, device=device)
+        mid_lse = torch.empty((rows, num_qo_heads), dtype=torch.float32, device=device)
+    return (
+        put(kv_entries),
+        put(vnodes[0]),
+        put(vnodes[1]),
+        put(q_entries),
+        put(vnodes[2]),
+        put(vnodes[3]),
+        put(per_request[0]),
+        put(per_request[1]),
+        put(per_request[2]),
+        mid_o,
+        mid_lse,
+        phase_nums,
+        phase_offs,
+    )
+
+
 def fasttree_preparation(
     tree_info,
     KV_ptrs,
@@ -502,81 +583,18 @@ def fasttree_preparation(
     also carries the program table, which ``fasttree_decode`` picks up; the programs are laid out
     for ``num_cus`` compute units (None: those ``device`` reports, 256 where it is not a GPU).
     """
-    import torch
-
-    from .launch_schedule import LaunchPhases, block_programs
-
     plan = fasttree_plan(
         tree_info, KV_ptrs, batch_size, num_kv_heads,
         KV_SPLIT_SIZES, para_threshs1, para_threshs2, params, kv_slot_map=kv_slot_map,
     )
 
-    names = iter(("vnode_to_kv_entries", "vnode_to_kv_offs", "vnode_to_kv_lens", "vnode_to_q_entries", "vnode_to_q_offs",
-                  "vnode_to_q_lens", "req_to_vnode_entries", "req_to_vnode_offs", "req_to_vnode_lens"))
-
-    def place(name, values):
-        if buffers is not None:
-            return buffers.fill(name, values)
-        host = torch.from_numpy(np.ascontiguousarray(np.asarray(values, dtype=np.int32)))
-        return host.to(device)
-
-    def put(values):
-        return place(next(names), values)  # (the nine arrays are placed in this order below)
-
-    rows = plan.num_rows
-    vnodes = (plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens)
-    q_entries = plan.vnode_to_q_entries
-    per_request = (plan.req_to_vnode_entries, plan.req_to_vnode_offs, plan.req_to_vnode_lens)
-    phase_nums, phase_offs = list(plan.phase_node_nums), list(plan.phase_node_offsets)
-    if launch_order:
-        group = max(1, num_qo_heads // num_kv_heads)
-        if num_cus is None:
-            from .launch_schedule import compute_units
-            num_cus = compute_units(device)
-        sched = block_programs(*vnodes, q_entries, batch_size, group, num_kv_heads, head_dim=head_dim, num_cus=num_cus)
-        vnodes = (sched.kv_offs, sched.kv_lens, sched.q_offs, sched.q_lens)
-        q_entries = sched.q_entries
-        per_request = (sched.req_entries, sched.req_offs, sched.req_lens)
-        rows = sched.num_rows
-        phase_nums, phase_offs = LaunchPhases(sched.phase_node_nums), list(sched.phase_node_offsets)
-        phase_nums.modelled_us, phase_nums.num_cus, phase_nums.block_slots = sched.modelled_us, sched.num_cus, sched.block_slots
-        if sched.num_programs > 0:
-            phase_nums.prog_table = place("prog_table", sched.prog_table.reshape(-1))
-            phase_nums.num_programs = sched.num_programs
-            phase_nums.narrow_in_programs = sched.narrow_in_programs
-        from . import launch_schedule
-        if sched.num_programs > 0 and head_dim >= 32 and launch_schedule.USE_PROGRAM_RECORDS:
-            records = launch_schedule.program_records(plan.vnode_to_kv_entries, *vnodes, q_entries, sched.prog_table,
-                                                      phase_offs[0], group)
-            phase_nums.prog_records = place("prog_records", records.reshape(-1))
-        if phase_nums[1] > 0 and head_dim >= 32 and launch_schedule.USE_NARROW_RECORDS:
-            from .launch_schedule import narrow_records
-            records = narrow_records(plan.vnode_to_kv_entries, *vnodes, q_entries, phase_offs[1], phase_nums[1])
-            phase_nums.narrow_table = place("narrow_table", records.reshape(-1))
-        if head_dim >= 32 and launch_schedule.USE_REQUEST_RECORDS:
-            from .launch_schedule import request_records
-            phase_nums.req_table = place("req_table", request_records(*per_request).reshape(-1))
-    if buffers is not None:
-        if rows > buffers.mid_o.shape[0] or buffers.mid_o.shape[1:] != (num_qo_heads, head_dim):
-            raise ValueError(f"the scratch of the buffers ({tuple(buffers.mid_o.shape)}) does not hold "
-                             f"{rows} rows of {num_qo_heads} x {head_dim}")
-        mid_o, mid_lse = buffers.mid_o[:rows], buffers.mid_lse[:rows]
-    else:
-        mid_o = torch.empty((rows, num_qo_heads, head_dim), dtype=torch.float32, device=device)
-        mid_lse = torch.empty((rows, num_qo_heads), dtype=torch.float32, device=device)
-    aux = (
-        put(plan.vnode_to_kv_entries),
-        put(vnodes[0]),
-        put(vnodes[1]),
-        put(q_entries),
-        put(vnodes[2]),
-        put(vnodes[3]),
-        put(per_request[0]),
-        put(per_request[1]),
-        put(per_request[2]),
-        mid_o,
-        mid_lse,
-        phase_nums,
-        phase_offs,
+    aux = place_plan(
+        plan.vnode_to_kv_entries,
+        (plan.vnode_to_kv_offs, plan.vnode_to_kv_lens, plan.vnode_to_q_offs, plan.vnode_to_q_lens),
+        plan.vnode_to_q_entries,
+        (plan.req_to_vnode_entries, plan.req_to_vnode_offs, plan.req_to_vnode_lens),
+        list(plan.phase_node_nums), list(plan.phase_node_offsets),
+        batch_size, num_qo_heads, num_kv_heads, head_dim,
+        device=device, launch_order=launch_order, buffers=buffers, num_cus=num_cus,
     )
     return aux, plan.node_assignments

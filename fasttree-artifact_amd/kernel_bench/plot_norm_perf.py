@@ -6,7 +6,7 @@ of bars per tree, every engine's speed divided by the fastest engine's of that t
 
 Reads the table ``run_benchmark.py`` writes (milliseconds per engine), so the engines are the
 ones measured here: the gathered decode without sharing, the naive plan, DeFT-Flatten (its own
-masked kernel), the node-wise (cascade-style) plan, the tree decode without the greedy merge, and the
+masked kernel), multi-level cascade attention, the tree decode without the greedy merge, and the
 tree decode.
 """
 import argparse
@@ -14,7 +14,7 @@ import argparse
 ENGINES = [("gathered ms", "Gathered (no sharing)", "#CCCCCC"),
            ("tree, naive ms", "Tree, naive", "#B4C7E7"),
            ("DeFT ms", "DeFT", "#FFE699"),
-           ("node-wise ms", "Node-wise (cascade)", "#F6CAE5"),
+           ("cascade ms", "Cascade", "#F6CAE5"),
            ("tree, w/o greedy ms", "Tree w/o greedy", "#F8CBAD"),
            ("tree ms", "Tree decode", "#C5796A")]
 

@@ -2,10 +2,10 @@
 its parse_output.py / plot_norm_perf.py derive: 15 level-regular trees x 3 head configurations;
 per case the gathered decode without sharing ("flash attn"), the tree decode, the two ablations
 of the tree decode (gamma = 10 with one KV split: every request its own full path, "naive";
-gamma = -10: never merge, "w/o greedy"), and the never-merge plan without KV splits
-("node-wise": every tree node one batched attention over its own KV, merged per request -- the
-schedule of a multi-level cascade attention, which the reference measures with FlashInfer,
-kernel_bench/bench_cascade.py), and DeFT-Flatten (subtrees of 128 tokens of the depth-first token
+gamma = -10: never merge, "w/o greedy"), multi-level cascade attention ("cascade": every tree
+node one batched attention over its own KV, merged per request -- bench_cascade.py here, the
+plan / run calls of the wrapper the reference measures with FlashInfer,
+kernel_bench/bench_cascade.py and run_benchmark.sh:83-88), and DeFT-Flatten (subtrees of 128 tokens of the depth-first token
 order, one block per subtree with a mask word per token, kernel_bench/DeFT.py) on its own kernel.
 
     python run_benchmark.py --out sweep --preset mi355x [--cases 0,8,9] [--heads "32 8"]
@@ -26,6 +26,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, HERE)
 
+import bench_cascade  # noqa: E402
 import benchmark  # noqa: E402
 import tree_generation  # noqa: E402
 
@@ -74,8 +75,6 @@ def run_case(out_dir, nodes, contexts, q_heads, k_heads, preset, log=print, extr
                           "--kv_split_sizes", "81920,81920", "--signature", "fasttree 10"]),
         ("no_greedy", base + ["--choice", "fasttree", "--alpha", "0", "--beta", "0", "--gamma", "-10",
                               "--signature", "fasttree -10"]),
-        ("node_wise", base + ["--choice", "fasttree", "--alpha", "0", "--beta", "0", "--gamma", "-10",
-                              "--kv_split_sizes", "81920,81920", "--signature", "fasttree node-wise"]),
     ]
     row = {"tree": f"{nodes} / {contexts}", "heads": f"{q_heads}/{k_heads}", "preset": preset}
     with open(out_path, "w") as fh:
@@ -96,22 +95,27 @@ def run_case(out_dir, nodes, contexts, q_heads, k_heads, preset, log=print, extr
                 row["measured_us"] = res.get("stage1_measured_us")
             else:
                 row[tag] = next(iter(v for k, v in res.items() if k.startswith("fasttree")), None)
+        text = io.StringIO()
+        with contextlib.redirect_stdout(text):
+            row["cascade"] = bench_cascade.main(["--node_num_per_level", nodes, "--node_seqlen_per_level", contexts,
+                                                 "--num_qo_heads", str(q_heads), "--num_kv_heads", str(k_heads)])["cascade"]
+        fh.write(text.getvalue())
     log(f"{row['tree']:60s} {row['heads']:6s} {preset:9s} gathered {row['flash_attn']:.4f} ms  tree {row['fasttree']:.4f} ms  "
-        f"naive {row['naive']:.4f}  w/o greedy {row['no_greedy']:.4f}  node-wise {row['node_wise']:.4f}  DeFT {row['deft']:.4f}  "
+        f"naive {row['naive']:.4f}  w/o greedy {row['no_greedy']:.4f}  cascade {row['cascade']:.4f}  DeFT {row['deft']:.4f}  "
         f"check {row['check']} / {row['deft_check']}  max abs {row['max_abs']:.1e}")
     return row
 
 
 def write_table(rows, path):
-    engines = ["flash_attn", "naive", "deft", "node_wise", "no_greedy", "fasttree"]
+    engines = ["flash_attn", "naive", "deft", "cascade", "no_greedy", "fasttree"]
     with open(path, "w") as fh:
-        fh.write("| tree (nodes / tokens per level) | q/kv heads | preset | gathered ms | tree, naive ms | DeFT ms | node-wise ms | tree, w/o greedy ms | tree ms | "
-                 "speed-up over gathered | normalised: gathered / naive / DeFT / node-wise / w/o greedy / tree | allclose 1e-2 | max abs | worst request mean abs |\n")
+        fh.write("| tree (nodes / tokens per level) | q/kv heads | preset | gathered ms | tree, naive ms | DeFT ms | cascade ms | tree, w/o greedy ms | tree ms | "
+                 "speed-up over gathered | normalised: gathered / naive / DeFT / cascade / w/o greedy / tree | allclose 1e-2 | max abs | worst request mean abs |\n")
         fh.write("|---|---|---|---|---|---|---|---|---|---|---|---|---|---|\n")
         for r in rows:
             best = min(r[e] for e in engines)
             norm = " / ".join(f"{best / r[e]:.2f}" for e in engines)
-            fh.write(f"| {r['tree']} | {r['heads']} | {r['preset']} | {r['flash_attn']:.4f} | {r['naive']:.4f} | {r['deft']:.4f} | {r['node_wise']:.4f} | {r['no_greedy']:.4f} | "
+            fh.write(f"| {r['tree']} | {r['heads']} | {r['preset']} | {r['flash_attn']:.4f} | {r['naive']:.4f} | {r['deft']:.4f} | {r['cascade']:.4f} | {r['no_greedy']:.4f} | "
                      f"{r['fasttree']:.4f} | {r['flash_attn'] / r['fasttree']:.2f} | {norm} | {'passed' if r['check'] and r['deft_check'] else 'FAILED'} | "
                      f"{r['max_abs']:.1e} | {r['mean_abs']:.1e} |\n")
         fh.write("\n")

@@ -65,7 +65,7 @@ def test_sweep_lists_and_table():
 
 
 def test_sweep_table_is_normalised_to_the_best_engine(tmp_path):
-    row = dict(tree="1,2 / 8,8", heads="32/8", preset="mi355x", flash_attn=0.4, naive=0.2, deft=0.125, node_wise=0.2, no_greedy=0.1,
+    row = dict(tree="1,2 / 8,8", heads="32/8", preset="mi355x", flash_attn=0.4, naive=0.2, deft=0.125, cascade=0.2, no_greedy=0.1,
                fasttree=0.05, check=True, deft_check=True, max_abs=1e-4, mean_abs=1e-5)
     path = tmp_path / "r.md"
     run_benchmark.write_table([row], str(path))
@@ -80,7 +80,7 @@ def test_plot_script_reads_the_sweep_table_and_draws_it(tmp_path):
     """plot_norm_perf.py takes the table run_benchmark.py writes: one row per case of the chosen
     preset, every engine column present, and a picture comes out."""
     import plot_norm_perf
-    rows = [dict(tree=f"1,{n} / 8,8", heads=h, preset=p, flash_attn=0.4, naive=0.2, deft=0.125, node_wise=0.2, no_greedy=0.1,
+    rows = [dict(tree=f"1,{n} / 8,8", heads=h, preset=p, flash_attn=0.4, naive=0.2, deft=0.125, cascade=0.2, no_greedy=0.1,
                  fasttree=0.05, check=True, deft_check=True, max_abs=1e-4, mean_abs=1e-5)
             for n in (2, 4) for h in ("16/1", "32/8") for p in ("reference", "mi355x")]
     table = tmp_path / "r.md"
