@@ -15,7 +15,6 @@ from helpers import bits16_to_tensor, kernel_golden, per_request_errors, planner
 ARRAYS = ["vnode_to_kv_entries", "vnode_to_kv_offs", "vnode_to_kv_lens", "vnode_to_q_entries", "vnode_to_q_offs",
           "vnode_to_q_lens", "req_to_vnode_entries", "req_to_vnode_offs", "req_to_vnode_lens", "node_assignments"]
 DTYPES = {"fp16": torch.float16, "bf16": torch.bfloat16}
-SMALL_PLANNER_CASES = [c for c in PLANNER_CASES if c["name"] != "c4" and not c["name"].startswith("c4_")]
 
 
 @pytest.fixture(scope="module")
@@ -23,7 +22,7 @@ def goldens():
     return planner_goldens()
 
 
-@pytest.mark.parametrize("case", SMALL_PLANNER_CASES, ids=[c["name"] for c in SMALL_PLANNER_CASES])
+@pytest.mark.parametrize("case", PLANNER_CASES, ids=[c["name"] for c in PLANNER_CASES])
 def test_plan_restatement_matches_reference_fixture(case, goldens):
     gold = goldens[case["name"]]
     tree, ptrs, batch = build_tree(case["tree"])
@@ -52,13 +51,14 @@ def test_two_stage_arithmetic_matches_reference_kernels(case):
     """mid_o, mid_lse and o of the restated arithmetic agree with what the reference's Triton
     kernels wrote (CPU interpreter) far inside the parity tolerance: only the summation
     order inside the dot products differs."""
-    if case["name"] == "k_c1" or case.get("keep_every"):
-        pytest.skip("the full-size cases are covered by the dense check below; the tile loop is slow in torch")
     tree, ptrs, batch, plan, q, k, v, gold = _kernel_case(case)
     sm_scale = 1.0 / math.sqrt(case["D"])
     o, mid_o, mid_lse = oracle.fasttree_decode_arith(q, k, v, plan, case["TSKs"][0], sm_scale)
-    assert torch.allclose(mid_lse, torch.from_numpy(gold["mid_lse"]), rtol=0, atol=2e-5)
-    assert torch.allclose(mid_o, torch.from_numpy(gold["mid_o"]), rtol=0, atol=2e-4 if case["dtype"] == "fp16" else 2e-3)
+    if "mid_o" in gold:      # (the full-size fixtures hold the outputs of a request subset only)
+        assert torch.allclose(mid_lse, torch.from_numpy(gold["mid_lse"]), rtol=0, atol=2e-5)
+        assert torch.allclose(mid_o, torch.from_numpy(gold["mid_o"]), rtol=0, atol=2e-4 if case["dtype"] == "fp16" else 2e-3)
+    if "requests" in gold:
+        o = o[gold["requests"].tolist()]
     want = bits16_to_tensor(gold["o"], DTYPES[case["dtype"]])
     worst_max, worst_mean = per_request_errors(o, want)
     one_ulp = 2e-3 if case["dtype"] == "fp16" else 1.6e-2      # outputs are O(1): half / bfloat16 spacing near 2
@@ -69,9 +69,8 @@ def test_two_stage_arithmetic_matches_reference_kernels(case):
 def test_arithmetic_for_sampled_requests_matches_reference_kernels(case):
     """decode_arith_for_requests (the two-stage arithmetic for a few requests of a plan, what the
     bfloat16 GPU cases are compared with like for like) against what the reference's own kernels
-    wrote for those requests, and, where the whole plan is cheap enough to evaluate, against
-    fasttree_decode_arith on the whole plan: restricting a plan to some of its requests changes
-    nothing for them."""
+    wrote for those requests, and against fasttree_decode_arith on the whole plan: restricting a
+    plan to some of its requests changes nothing for them."""
     tree, ptrs, batch, plan, q, k, v, gold = _kernel_case(case)
     sm_scale = 1.0 / math.sqrt(case["D"])
     kept = gold["requests"].tolist() if "requests" in gold else list(range(batch))
@@ -83,10 +82,9 @@ def test_arithmetic_for_sampled_requests_matches_reference_kernels(case):
     worst_max, worst_mean = per_request_errors(o, want[picks])
     one_ulp = 2e-3 if case["dtype"] == "fp16" else 1.6e-2
     assert worst_max <= one_ulp and worst_mean <= one_ulp / 20
-    if case["name"] != "k_c1" and not case.get("keep_every"):
-        full, _, _ = oracle.fasttree_decode_arith(q, k, v, plan, case["TSKs"][0], sm_scale)
-        assert torch.allclose(o.float(), full[sample].float(), rtol=0, atol=1e-3 if case["dtype"] == "fp16" else 8e-3)
-        assert (o.float() - full[sample].float()).abs().mean() <= 2e-5
+    full, _, _ = oracle.fasttree_decode_arith(q, k, v, plan, case["TSKs"][0], sm_scale)
+    assert torch.allclose(o.float(), full[sample].float(), rtol=0, atol=1e-3 if case["dtype"] == "fp16" else 8e-3)
+    assert (o.float() - full[sample].float()).abs().mean() <= 2e-5
 
 
 @pytest.mark.parametrize("case", KERNEL_CASES, ids=[c["name"] for c in KERNEL_CASES])
