@@ -58,8 +58,8 @@ import numpy as np
 
 #: Query rows one block of the first-stage kernel serves per pass (4 waves x 32 rows).
 BLOCK_ROWS = 128
-#: Blocks and waves of the first-stage kernel one compute unit holds at a time (72 KB of LDS and
-#: 238 registers per block of four waves).
+#: Blocks and waves of the first-stage kernel one compute unit holds at a time (73 KB of LDS and
+#: 241 registers per wave of a block of four).
 BLOCKS_PER_CU = 2
 WAVES_PER_CU = 8
 #: Compute units assumed when no device can be asked (an MI355X has 256).
